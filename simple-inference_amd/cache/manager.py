@@ -20,7 +20,8 @@ rows of a replayed graph write there.
 A group with a window keeps, for each request, only pages that a future query
 can still see: before a step that starts at position ``s``, pages that lie wholly
 below ``s - window + 1`` go back to the allocator, and their table entries
-become -1.
+become -1.  A group whose queries see only their own block of ``chunk`` positions
+does the same with the pages below the start of the block that holds ``s``.
 
 Beside the pages there are *slots*: one row of fixed size per running request
 and per stateful run of a layer, set to the state's initial value when a request gets its slot.  The
@@ -72,11 +73,12 @@ class PagedGroup:
     def pages_to_reserve(self, total_tokens: int, max_chunk: int) -> int:
         """Most pages a request of ``total_tokens`` holds at once, fed at most ``max_chunk`` a step."""
         full = pages_for(total_tokens, self.page_size)
-        if self.need.window is None:
+        if self.need.span is None:
             return full
         # A step sees keys from (start - window + 1) to (start + chunk - 1): window + chunk - 1
         # positions, which touch at most that many / page_size pages plus one for misalignment.
-        span = self.need.window + max_chunk - 1
+        # (A block of positions in place of the window: from the block's start, at most as far back.)
+        span = self.need.span + max_chunk - 1
         return min(full, pages_for(span, self.page_size) + 1)
 
     def begin(self, req: int, reserve: int) -> None:
@@ -87,8 +89,8 @@ class PagedGroup:
     def extend(self, req: int, start: int, end: int) -> None:
         """Makes the table ready for a step that writes positions ``start .. end-1``."""
         table = self.tables[req]
-        if self.need.window is not None:
-            first_visible = max(0, start - self.need.window + 1)
+        if self.need.span is not None:
+            first_visible = self.need.first_visible(start)
             for idx in range(min(first_visible // self.page_size, len(table))):
                 if table[idx] >= 0:
                     self.pool.drop(req, table[idx], restore_promise=True)
@@ -183,7 +185,7 @@ class CacheManager:
         if req in self.lengths:
             raise ValueError(f"request {req} is already admitted")
         shared = list(shared_pages or [])
-        if shared and (len(self.groups) != 1 or self.groups[0].need.window is not None or self.layout.states):
+        if shared and (len(self.groups) != 1 or self.groups[0].need.span is not None or self.layout.states):
             raise ValueError("shared prefix pages need exactly one group without a window and no state")
         if not self.can_admit(total_tokens, max_chunk, len(shared)):
             raise MemoryError(f"cannot admit request {req}: no slot or not enough pages")

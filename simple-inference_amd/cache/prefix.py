@@ -49,7 +49,7 @@ class PrefixCache:
     def __init__(self, cache, max_pages: int):
         if max_pages <= 0:
             raise ValueError(f"max_pages must be positive, got {max_pages}")
-        if len(cache.groups) != 1 or cache.groups[0].need.window is not None or cache.layout.states:
+        if len(cache.groups) != 1 or cache.groups[0].need.span is not None or cache.layout.states:
             raise ValueError("prefix reuse needs one cache group without a window and no per-request state")
         self.pool = cache.groups[0].pool
         self.page_size = cache.page_size

@@ -1,6 +1,7 @@
 """One registry from an architecture's name to the code that builds its model.
 
-config.json names the architecture in ``architectures[0]``.  An entry holds two
+config.json names the architecture in ``architectures[0]`` (or, in the configurations that
+name one design as a plain string, in ``architecture``).  An entry holds two
 functions: ``parse_config`` turns the json dictionary into the architecture's
 typed configuration, and ``build_plan`` turns that configuration into a
 ``ModelPlan`` (the list of layers, their parts, their weights' names, their
@@ -58,10 +59,17 @@ def get_architecture(name: str) -> Architecture:
 
 
 def architecture_of(config_dict: Mapping[str, Any]) -> Architecture:
-    """The entry that ``config.json``'s ``architectures[0]`` names."""
+    """The entry that ``config.json``'s ``architectures[0]`` (or its ``architecture``) names."""
+    return get_architecture(architecture_name(config_dict))
+
+
+def architecture_name(config_dict: Mapping[str, Any]) -> str:
     archs = config_dict.get("architectures")
-    if not archs:
-        raise UnknownArchitecture(
-            "config.json has no 'architectures' entry; known: " + ", ".join(known_architectures())
-        )
-    return get_architecture(archs[0])
+    if archs:
+        return str(archs[0])
+    single = config_dict.get("architecture")
+    if isinstance(single, str) and single:
+        return single
+    raise UnknownArchitecture(
+        "config.json has no 'architectures' entry; known: " + ", ".join(known_architectures())
+    )

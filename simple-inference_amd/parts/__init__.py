@@ -5,7 +5,7 @@ from .registry import (
     register_position_encoding,
 )
 from .context import BuildEnv, LayerCache, ResidualStream, StepContext
-from . import norm, rope, attention, swiglu, block, embedding  # noqa: F401  (registers the built-in kinds)
+from . import norm, rope, attention, swiglu, dense, block, embedding  # noqa: F401  (registers the built-in kinds)
 from .model import DecoderModel
 
 __all__ = [

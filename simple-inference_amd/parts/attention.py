@@ -12,6 +12,19 @@ scale applied after the dot; key ``j`` is visible to a query at position ``p`` i
 The three projections are stacked into one ``[(Hq + 2 Hkv) D, H]`` matrix at load.
 A mixer whose ``kv_from_layer`` is set projects only q and reads the pages that
 the named layer's latest run wrote.
+
+Further forms, each switched on by a parameter of its own and free to combine:
+
+* ``value_head_dim``: value heads of another width ``Dv`` than the keys'; the stacked matrix is then
+  ``[Hq D + Hkv D + Hkv Dv, H]`` and the output projection takes ``Hq Dv`` columns.
+* ``bias``: q, k and v have biases, added to the projections before anything else.
+* ``qk_norm`` (``{"eps": e}``): every q and k head is divided by its root mean square over the head
+  (``x / sqrt(mean(x^2) + e)``) and multiplied by a gain of size ``D`` that all heads share (one for q, one for k),
+  after the bias and before the rotation.
+* ``chunk``: position ``p`` sees key ``j <= p`` only if both lie in the same block of ``chunk`` positions, blocks
+  counted from position 0 of the sequence.
+* ``sink``: one learned number per query head joins the softmax's denominator as ``exp(sink_h)``; it has no key,
+  no value and is not scaled.
 """
 
 from __future__ import annotations
@@ -34,7 +47,8 @@ def _shared_position_encoding(spec, env):
 @register_mixer("attention")
 class Attention:
     """params: hidden_size, num_heads, num_kv_heads, head_dim, position
-    (``{"kind", "params"}``), and optionally window, scale, kv_from_layer."""
+    (``{"kind", "params"}``), and optionally window, scale, kv_from_layer, value_head_dim, bias, qk_norm, chunk,
+    sink."""
 
     def __init__(self, params, env):
         self.hidden = int(params["hidden_size"])
@@ -51,15 +65,28 @@ class Attention:
         scale = params.get("scale")
         self.scale = float(scale) if scale is not None else 1.0 / (self.head_dim ** 0.5)
         self.kv_from_layer = params.get("kv_from_layer")
+        self.value_dim = int(params.get("value_head_dim") or self.head_dim)
+        self.bias = bool(params.get("bias", False))
+        qk_norm = params.get("qk_norm")
+        self.qk_norm_eps = float(qk_norm["eps"]) if qk_norm else None
+        self.chunk = params.get("chunk")
+        if self.chunk is not None:
+            self.chunk = int(self.chunk)
+            if self.chunk <= 0:
+                raise ValueError(f"chunk must be positive, got {self.chunk}")
+        self.sink = bool(params.get("sink", False))
+        if self.kv_from_layer is not None and (self.bias or self.qk_norm_eps is not None or self.value_dim != self.head_dim):
+            raise ValueError("a mixer that reads another layer's keys and values has plain q heads of the keys' width")
         self.position = _shared_position_encoding(params.get("position", {"kind": "none", "params": {}}), env)
         if self.position.rotary_dim > self.head_dim:
             raise ValueError(f"rotary_dim {self.position.rotary_dim} exceeds head_dim {self.head_dim}")
         check = getattr(env.kernels, "check_attention_geometry", None)
         if check is not None:     # sizes the kernels refuse are refused here, when the model is built
-            check(self.num_heads, self.num_kv_heads, self.head_dim)
+            check(self.num_heads, self.num_kv_heads, max(self.head_dim, self.value_dim))
         self.env = env
         self.w_qkv = None
         self.w_o = None
+        self.b_qkv = self.q_gain = self.k_gain = self.sinks = None
 
     takes_scaled_rows = True   # the input goes to ``qkv_to_cache`` only
 
@@ -70,10 +97,18 @@ class Attention:
     def weight_specs(self):
         q = self.num_heads * self.head_dim
         kv = self.num_kv_heads * self.head_dim
-        specs = {"q": TensorSpec((q, self.hidden)), "o": TensorSpec((self.hidden, q))}
+        v = self.num_kv_heads * self.value_dim
+        specs = {"q": TensorSpec((q, self.hidden)), "o": TensorSpec((self.hidden, self.num_heads * self.value_dim))}
         if self.writes_kv:
             specs["k"] = TensorSpec((kv, self.hidden))
-            specs["v"] = TensorSpec((kv, self.hidden))
+            specs["v"] = TensorSpec((v, self.hidden))
+        if self.bias:
+            specs.update({"q_bias": TensorSpec((q,), "vector"), "k_bias": TensorSpec((kv,), "vector"),
+                          "v_bias": TensorSpec((v,), "vector")})
+        if self.qk_norm_eps is not None:
+            specs.update({"q_norm": TensorSpec((self.head_dim,), "vector"), "k_norm": TensorSpec((self.head_dim,), "vector")})
+        if self.sink:
+            specs["sink"] = TensorSpec((self.num_heads,), "vector")
         return specs
 
     def bind(self, tensors):
@@ -82,6 +117,12 @@ class Attention:
         else:
             self.w_qkv = tensors["q"].contiguous()
         self.w_o = tensors["o"].contiguous()
+        if self.bias:
+            self.b_qkv = torch.cat([tensors["q_bias"], tensors["k_bias"], tensors["v_bias"]]).contiguous()
+        if self.qk_norm_eps is not None:
+            self.q_gain, self.k_gain = tensors["q_norm"].contiguous(), tensors["k_norm"].contiguous()
+        if self.sink:
+            self.sinks = tensors["sink"].contiguous()
         prepare = getattr(self.env.kernels, "prepare_pending_weight", None)
         if prepare is not None:   # the kernels may keep a copy of their own of a weight whose product is left pending
             prepare(self.w_o)
@@ -89,7 +130,7 @@ class Attention:
     def plain_form(self):
         """What this mixer is, as plain data, for kernels that can run a whole block in one call; None for the forms
         that only ``forward`` covers (reading another layer's keys and values)."""
-        if not self.writes_kv or type(self).forward is not Attention.forward:
+        if not self.writes_kv or type(self).forward is not Attention.forward or self._options():
             return None     # a subclass with a forward of its own is no longer what this form describes
         cos, sin = self.position.tables()
         return {"kind": "paged_attention", "w_qkv": self.w_qkv, "w_o": self.w_o, "hidden": self.hidden,
@@ -97,8 +138,14 @@ class Attention:
                 "rotary_dim": self.position.rotary_dim, "cos": cos, "sin": sin, "scale": self.scale,
                 "window": self.window}
 
+    def _options(self) -> bool:
+        """Whether any of the further forms is switched on (the kernels then get them as keyword arguments)."""
+        return (self.bias or self.qk_norm_eps is not None or self.sink or self.chunk is not None
+                or self.value_dim != self.head_dim)
+
     def cache_need(self):
-        return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window)
+        return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window,
+                           self.value_dim if self.value_dim != self.head_dim else None, self.chunk)
 
     def state_need(self):
         return None
@@ -106,9 +153,21 @@ class Attention:
     def forward(self, h, ctx, cache):
         k = self.env.kernels
         cos, sin = self.position.tables()
+        project, attend = {}, {}
+        if self._options():   # only then: a kernels object that knows none of these forms serves the plain mixer
+            if self.value_dim != self.head_dim:
+                project["value_dim"] = attend["value_dim"] = self.value_dim
+            if self.bias:
+                project["bias"] = self.b_qkv
+            if self.qk_norm_eps is not None:
+                project["qk_norm"] = (self.q_gain, self.k_gain, self.qk_norm_eps)
+            if self.chunk is not None:
+                attend["chunk"] = self.chunk
+            if self.sink:
+                attend["sinks"] = self.sinks
         qkv = k.qkv_to_cache(
             h, self.w_qkv, self.num_heads, self.num_kv_heads if self.writes_kv else 0, self.head_dim,
-            self.position.rotary_dim, cos, sin, ctx, cache)
+            self.position.rotary_dim, cos, sin, ctx, cache, **project)
         out = k.paged_attention(
-            qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window, ctx, cache)
+            qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window, ctx, cache, **attend)
         return k.pending_linear(out, self.w_o)   # the norm after it may have it added into the residual

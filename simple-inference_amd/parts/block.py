@@ -4,6 +4,11 @@ Pre-norm (reference: ``model/block.py:135-147``):
 ``x += mixer(norm1(x))``; ``x += feed_forward(norm2(x))``.  Each add is carried
 as the stream's pending delta and summed into the float32 residual by the norm
 that follows (the next layer's, or the model's last norm).
+
+Output-norm: ``x += norm1(mixer(x))``; ``x += norm2(feed_forward(x))``.  The sublayers read the residual itself
+(rounded to the compute dtype) and the norm sits on what a sublayer returns; the kernel that adds the normed
+output into the float32 residual also leaves the rounded residual for the next sublayer.  A layer of this kind
+may have no feed-forward.
 """
 
 from __future__ import annotations
@@ -48,3 +53,26 @@ def _normed(norm, consumer, stream):
     if getattr(norm, "gives_scaled_rows", False) and getattr(consumer, "takes_scaled_rows", False):
         return norm.forward(stream, scaled_ok=True)
     return norm.forward(stream)
+
+
+@register_block("output_norm")
+class OutputNormBlock:
+    def __init__(self, mixer, mixer_norm, feed_forward=None, feed_forward_norm=None):
+        if (feed_forward is None) != (feed_forward_norm is None):
+            raise ValueError("an output-norm block has a feed-forward and its norm, or neither")
+        self.mixer = mixer
+        self.mixer_norm = mixer_norm
+        self.feed_forward = feed_forward
+        self.feed_forward_norm = feed_forward_norm
+
+    def forward(self, stream, ctx, cache):
+        if stream.raw_delta is not None:
+            raise NotImplementedError("an output-norm block cannot follow a block that leaves its sum to the next norm")
+        x = stream.lowered
+        if x is None:    # the first block of a step, or the residual is already of the compute dtype
+            x = stream.residual
+            if x.dtype != self.mixer_norm.env.dtype:
+                x = ctx.kernels.cast(x, self.mixer_norm.env.dtype)
+        x = self.mixer_norm.add_normed(stream, self.mixer.forward(x, ctx, cache))
+        if self.feed_forward is not None:
+            self.feed_forward_norm.add_normed(stream, self.feed_forward.forward(x, ctx))

@@ -71,13 +71,17 @@ class ResidualStream:
     A part may leave its last product uncomputed (an object with ``compute()``, as the kernels'
     ``pending_linear`` returns): ``raw_delta`` shows it to a norm that can have it computed
     straight into the residual; ``delta`` computes it for everybody else.
+
+    ``lowered`` is the residual in the compute dtype, if the kernel that last changed the residual left it (a
+    sublayer that reads the residual itself, not a norm of it, takes it from there); setting a delta forgets it.
     """
 
-    __slots__ = ("residual", "raw_delta")
+    __slots__ = ("residual", "raw_delta", "lowered")
 
     def __init__(self, residual: torch.Tensor, delta: Optional[torch.Tensor] = None):
         self.residual = residual
         self.raw_delta = delta
+        self.lowered = None
 
     @property
     def delta(self):
@@ -88,3 +92,5 @@ class ResidualStream:
     @delta.setter
     def delta(self, value):
         self.raw_delta = value
+        if value is not None:
+            self.lowered = None

@@ -1,6 +1,7 @@
 """Token embedding and output head (reference: ``ops/embedding.py:49-92``).
 
-The embedding gathers rows of ``[V, H]`` into the float32 residual.  The head is
+The embedding gathers rows of ``[V, H]`` into the float32 residual, multiplied by ``scale`` if its params give one
+(the product is taken in float32 on the stored row).  The head is
 ``logits = h E^T``; tied, it uses the embedding's storage (reference:
 ``ops/embedding.py:78-86``); untied, it has a matrix of its own, which the
 reference mishandles by overwriting the embedding (``model/llama.py:147-154``).
@@ -15,9 +16,12 @@ from .registry import register_embedding, register_head
 
 @register_embedding("embedding")
 class TokenEmbedding:
+    """params: vocab_size, hidden_size, and optionally scale (every gathered row is multiplied by it)."""
+
     def __init__(self, params, env):
         self.vocab = int(params["vocab_size"])
         self.hidden = int(params["hidden_size"])
+        self.scale = float(params.get("scale", 1.0))
         self.env = env
         self.weight = None
 
@@ -28,6 +32,8 @@ class TokenEmbedding:
         self.weight = tensors["weight"]
 
     def forward(self, ctx):
+        if self.scale != 1.0:
+            return self.env.kernels.embed(ctx.token_ids, self.weight, scale=self.scale)
         return self.env.kernels.embed(ctx.token_ids, self.weight)
 
 

@@ -3,6 +3,9 @@
 ``y = x * rsqrt(mean(x^2) + eps) * w`` with the statistic, the normalisation and
 the gain in float32 and one rounding to the compute dtype, as the reference's
 fused kernel does.  The add of the pending residual delta is fused in front.
+
+The same norm can sit behind a sublayer instead of in front of it (``add_normed``): the residual then grows by
+the norm of what the sublayer returned, ``x += y * rsqrt(mean(y^2) + eps) * w``, statistic and sum in float32.
 """
 
 from __future__ import annotations
@@ -33,6 +36,15 @@ class RMSNorm:
         if type(self).forward is not RMSNorm.forward:
             return None
         return {"kind": "rmsnorm", "weight": self.weight, "eps": self.eps, "size": self.size}
+
+    def add_normed(self, stream, y):
+        """``stream.residual += norm(y)``, in one kernel; returns the new residual in the compute dtype (the input
+        of the next sublayer), which the stream also keeps as ``lowered``."""
+        if hasattr(y, "compute"):     # a product left pending for a norm in front of the next sublayer: not this one
+            y = y.compute()
+        out = self.env.kernels.norm_add(stream.residual, y, self.weight, self.eps, self.env.dtype)
+        stream.lowered = out
+        return out
 
     def forward(self, stream, rows=None, scaled_ok=False):
         """Adds ``stream.delta`` into ``stream.residual`` and returns the normed rows.

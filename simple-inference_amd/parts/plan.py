@@ -117,7 +117,9 @@ class TensorSpec:
 
 @dataclass(frozen=True)
 class PagedKVNeed:
-    """Keys and values in pages: all keys (``window`` None) or the last ``window``.
+    """Keys and values in pages: all keys (``window`` and ``chunk`` None), the last ``window``, or those of the
+    current block of ``chunk`` positions (blocks counted from position 0: a query at ``p`` sees nothing below
+    ``p - p % chunk``).
 
     A page holds, per key/value head, ``page_size`` key rows of ``head_dim`` elements and as many value rows of
     ``value_head_dim`` elements (None: the same width).  The cache manager only stores them; what a row means is
@@ -128,6 +130,22 @@ class PagedKVNeed:
     head_dim: int
     window: Optional[int] = None
     value_head_dim: Optional[int] = None
+    chunk: Optional[int] = None
+
+    def first_visible(self, position: int) -> int:
+        """The oldest position that a query at ``position`` (or any later one) can still see."""
+        lo = 0
+        if self.window is not None:
+            lo = max(lo, position - self.window + 1)
+        if self.chunk is not None:
+            lo = max(lo, position - position % self.chunk)
+        return lo
+
+    @property
+    def span(self) -> Optional[int]:
+        """Most positions a query sees (None: no bound)."""
+        bounds = [b for b in (self.window, self.chunk) if b is not None]
+        return min(bounds) if bounds else None
 
     @property
     def value_dim(self) -> int:

@@ -15,6 +15,7 @@ import torch
 from .cache.manager import CacheManager
 from .config.engine_config import EngineConfig
 from .config.model_config import read_config_json
+from .config.registry import architecture_name
 from .engine.build import default_kernels, model_from_folder
 from .engine.step import StepEntry, StepRunner
 
@@ -33,7 +34,7 @@ class TraceReplayer:
             device=device, dtype=dtype, block_size=page, num_kv_blocks=num_pages, max_running=max_live,
             max_seq_len=min(max_pos, max(max_tokens, page)))
         self.kernels = kernels if kernels is not None else default_kernels()
-        self.architecture = (cfg.get("architectures") or ["?"])[0]
+        self.architecture = architecture_name(cfg)
         self.model, self.model_cfg = model_from_folder(model_folder, self.engine_cfg, self.kernels)
         self.cache = CacheManager(
             self.model.cache_layout(), page_size=page, num_pages=num_pages, max_running=max_live,

@@ -22,8 +22,17 @@ class TwinKernels:
     def place_tokens(self, token_ids, dst_rows, src_tokens, src_rows):
         token_ids[dst_rows.long()] = src_tokens[src_rows.long()]
 
-    def embed(self, token_ids, table):
-        return table[token_ids.long()].float()
+    def embed(self, token_ids, table, scale=1.0):
+        return table[token_ids.long()].float() * scale
+
+    def cast(self, x, dtype):
+        return x.to(dtype)
+
+    # -- residual += rms norm of a sublayer's output ---------------------------
+    def norm_add(self, residual, y, weight, eps, out_dtype):
+        yf = y.float()
+        residual.add_(yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps) * weight.float())
+        return residual if out_dtype == torch.float32 else residual.to(out_dtype)
 
     # -- residual add + rms norm ---------------------------------------------
     def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None):
@@ -54,16 +63,38 @@ class TwinKernels:
         g, u = gu[:, :inter].float(), gu[:, inter:].float()
         return (g * torch.sigmoid(g) * u).to(gu.dtype)
 
-    def qkv_to_cache(self, x, w_qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache):
+    def activated_linear(self, x, w, activation):
+        z = self.linear(x, w).float()
+        if activation == "relu2":
+            a = torch.relu(z) ** 2
+        elif activation == "gelu_tanh":
+            a = 0.5 * z * (1 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3)))
+        else:
+            raise ValueError(activation)
+        return a.to(x.dtype)
+
+    def qkv_to_cache(self, x, w_qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache,
+                     value_dim=None, bias=None, qk_norm=None):
         qkv = self.linear(x, w_qkv)
-        self.rope_kv_write(qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache)
+        self.rope_kv_write(qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache,
+                           value_dim=value_dim, bias=bias, qk_norm=qk_norm)
         return qkv
 
     # -- rotation + cache write ----------------------------------------------
-    def rope_kv_write(self, qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache):
+    def rope_kv_write(self, qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache,
+                      value_dim=None, bias=None, qk_norm=None):
         N = qkv.shape[0]
         pos = ctx.positions.long()
+        value_dim = value_dim or head_dim
+        if bias is not None:
+            qkv.copy_((qkv.float() + bias.float()).to(qkv.dtype))
         q = qkv[:, :n_heads * head_dim].view(N, n_heads, head_dim)
+
+        def normed(x, gain):
+            if qk_norm is None:
+                return x
+            xf = x.float()
+            return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + qk_norm[2]) * gain.float()).to(x.dtype)
 
         def rotate(x):
             if rotary_dim == 0:
@@ -78,13 +109,14 @@ class TwinKernels:
             out[..., half:rotary_dim] = b * c + a * s
             return out.to(x.dtype)
 
-        q.copy_(rotate(q))
+        q.copy_(rotate(normed(q, qk_norm[0] if qk_norm else None)))
         if n_kv_written == 0:
             return
         kv0 = n_heads * head_dim
         k = qkv[:, kv0:kv0 + n_kv_written * head_dim].view(N, n_kv_written, head_dim)
-        v = qkv[:, kv0 + n_kv_written * head_dim:kv0 + 2 * n_kv_written * head_dim].view(N, n_kv_written, head_dim)
-        k = rotate(k)
+        v0 = kv0 + n_kv_written * head_dim
+        v = qkv[:, v0:v0 + n_kv_written * value_dim].view(N, n_kv_written, value_dim)
+        k = rotate(normed(k, qk_norm[1] if qk_norm else None))
         ps = cache.page_size
         seq = ctx.seq_of_token.long()
         page = cache.block_table.long()[seq, pos // ps]
@@ -93,10 +125,12 @@ class TwinKernels:
         cache.v_pages[page, :, :, off] = v
 
     # -- attention over the pages --------------------------------------------
-    def paged_attention(self, qkv, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache):
+    def paged_attention(self, qkv, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache, value_dim=None,
+                        chunk=None, sinks=None):
         N = qkv.shape[0]
+        value_dim = value_dim or head_dim
         q = qkv[:, :n_heads * head_dim].view(N, n_heads, head_dim).float()
-        out = torch.zeros(N, n_heads, head_dim, dtype=torch.float32, device=qkv.device)
+        out = torch.zeros(N, n_heads, value_dim, dtype=torch.float32, device=qkv.device)
         ps = cache.page_size
         group = n_heads // n_kv_heads
         cu = ctx.cu_q.tolist()
@@ -108,6 +142,8 @@ class TwinKernels:
             first = kv_len[s] - (cu[s + 1] - cu[s])
             if window is not None:
                 lo = max(0, first - window + 1)
+            if chunk is not None:
+                lo = max(lo, first - first % chunk)
             idx = torch.arange(lo, L, device=qkv.device)
             pages = table[s, idx // ps]
             k = cache.k_pages[pages, :, idx % ps, :].float()          # [T, Hkv, D]
@@ -117,11 +153,17 @@ class TwinKernels:
             visible = idx[None, :] <= qpos[:, None]
             if window is not None:
                 visible &= idx[None, :] > qpos[:, None] - window
+            if chunk is not None:
+                visible &= idx[None, :] // chunk == qpos[:, None] // chunk
             for h in range(n_heads):
                 sc = (qs[:, h] @ k[:, h // group].T) * scale
                 sc = sc.masked_fill(~visible, float("-inf"))
-                out[cu[s]:cu[s + 1], h] = torch.softmax(sc, -1) @ v[:, h // group]
-        return out.view(N, n_heads * head_dim).to(qkv.dtype)
+                if sinks is not None:    # one more term in the denominator: a column whose value is nothing
+                    sc = torch.cat([sc, sinks[h].float().expand(sc.shape[0], 1)], dim=-1)
+                    out[cu[s]:cu[s + 1], h] = torch.softmax(sc, -1)[:, :-1] @ v[:, h // group]
+                else:
+                    out[cu[s]:cu[s + 1], h] = torch.softmax(sc, -1) @ v[:, h // group]
+        return out.view(N, n_heads * value_dim).to(qkv.dtype)
 
     # -- sampling --------------------------------------------------------------
     def sample(self, logits, temperature, top_k, top_p, uniform, all_greedy=False, filters=None):
