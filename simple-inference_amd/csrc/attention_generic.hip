@@ -8,9 +8,13 @@
 // rows of the batch, or on which pages hold the keys.
 //
 //   s_j = (q . k_j) * scale                                   scale after the dot
-//   visible: j <= pos, and j > pos - window if window > 0
+//   visible: j <= pos, and j > pos - window if window > 0, and j >= pos - pos % chunk if chunk > 0
+//            (blocks of chunk positions counted from position 0: a query sees its own block only)
 //   online softmax over chunks: m' = max(m, max_j s_j); p_j = exp(s_j - m');
 //   l = l * exp(m - m') + sum_j p_j;  acc = acc * exp(m - m') + sum_j p_j v_j;  o = acc / l
+//   with sinks: l += exp(sink_h - m) at the end, one learned number per query head that has no key and no
+//   value and is not scaled
+// Values may have another width (value_dim) than keys and queries (head_dim).
 // (reference: kernels/attention_kernel.py:184-251, :516-586).  Everything is float.
 #include "common.h"
 
@@ -21,7 +25,7 @@ __global__ __launch_bounds__(SIA_WAVE) void attention_generic_kernel(
     const T* __restrict__ q, int q_row_stride, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ seq_of_token,
     const int* __restrict__ positions, T* __restrict__ out, int n_heads, int n_kv, int head_dim,
-    int page_size, float scale, int window) {
+    int value_dim, int page_size, float scale, int window, int chunk, const float* __restrict__ sinks) {
     __shared__ float q_s[ATTN_MAX_HEAD_DIM];
     __shared__ float p_s[SIA_WAVE];
     __shared__ int page_s[SIA_WAVE];
@@ -30,7 +34,8 @@ __global__ __launch_bounds__(SIA_WAVE) void attention_generic_kernel(
     const int seq = seq_of_token[n];
     const int pos = positions[n];
     const int hk = h / (n_heads / n_kv);
-    const int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    if (chunk > 0) lo = max(lo, pos - pos % chunk);
     const int* table = block_table + (size_t)seq * table_width;
 
     const T* q_row = q + (size_t)n * q_row_stride + h * head_dim;
@@ -64,11 +69,11 @@ __global__ __launch_bounds__(SIA_WAVE) void attention_generic_kernel(
 #pragma unroll
         for (int dd = 0; dd < ATTN_MAX_HEAD_DIM / SIA_WAVE; ++dd) {
             const int d = lane + dd * SIA_WAVE;
-            if (d < head_dim) {
+            if (d < value_dim) {
                 float a = acc[dd] * alpha;
                 for (int jj = j_first; jj <= j_last; ++jj) {
                     if (page_s[jj] < 0) continue;
-                    const T* vp = v_pages + (((size_t)page_s[jj] * n_kv + hk) * head_dim + d) * page_size +
+                    const T* vp = v_pages + (((size_t)page_s[jj] * n_kv + hk) * value_dim + d) * page_size +
                                   ((c0 + jj) % page_size);
                     a += p_s[jj] * to_float(*vp);
                 }
@@ -78,12 +83,13 @@ __global__ __launch_bounds__(SIA_WAVE) void attention_generic_kernel(
         __syncthreads();
     }
 
-    T* o = out + ((size_t)n * n_heads + h) * head_dim;
+    T* o = out + ((size_t)n * n_heads + h) * value_dim;
+    if (sinks) l += expf(sinks[h] - m);   // m is finite: a token always sees itself
     const float inv = 1.f / l;
 #pragma unroll
     for (int dd = 0; dd < ATTN_MAX_HEAD_DIM / SIA_WAVE; ++dd) {
         const int d = lane + dd * SIA_WAVE;
-        if (d < head_dim) o[d] = from_float<T>(acc[dd] * inv);
+        if (d < value_dim) o[d] = from_float<T>(acc[dd] * inv);
     }
 }
 
@@ -93,17 +99,17 @@ SIA_EXPORT int sia_attention_max_head_dim() { return ATTN_MAX_HEAD_DIM; }
 SIA_EXPORT int sia_attention_generic(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
                                      const int* block_table, int table_width, const int* seq_of_token,
                                      const int* positions, void* out, int n_tokens, int n_heads, int n_kv,
-                                     int head_dim, int page_size, float scale, int window, int dtype,
-                                     hipStream_t stream) {
+                                     int head_dim, int value_dim, int page_size, float scale, int window, int chunk,
+                                     const float* sinks, int dtype, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
-    if (head_dim <= 0 || head_dim > ATTN_MAX_HEAD_DIM || n_kv <= 0 || n_heads % n_kv || page_size <= 0 ||
+    if (head_dim <= 0 || head_dim > ATTN_MAX_HEAD_DIM || value_dim <= 0 || value_dim > ATTN_MAX_HEAD_DIM || n_kv <= 0 || n_heads % n_kv || page_size <= 0 ||
         n_heads > 65535)
         return SIA_BAD_ARGUMENT;
     dim3 grid(n_tokens, n_heads), block(SIA_WAVE);
 #define LAUNCH(T)                                                                                              \
     hipLaunchKernelGGL(attention_generic_kernel<T>, grid, block, 0, stream, (const T*)q, q_row_stride,         \
                        (const T*)k_pages, (const T*)v_pages, block_table, table_width, seq_of_token, positions, \
-                       (T*)out, n_heads, n_kv, head_dim, page_size, scale, window)
+                       (T*)out, n_heads, n_kv, head_dim, value_dim, page_size, scale, window, chunk, sinks)
     if (dtype == SIA_F32) LAUNCH(float);
     else if (dtype == SIA_BF16) LAUNCH(bf16_t);
     else return SIA_BAD_ARGUMENT;

@@ -70,6 +70,20 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 constexpr float LOG2E = 1.4426950408889634f;
 
+// The oldest key a query at `pos` sees: all (window = chunk = 0), the last `window`, and/or those of its own block
+// of `chunk` positions (blocks counted from position 0).  It never falls as pos grows.
+__device__ __forceinline__ int first_visible(int pos, int window, int chunk) {
+    int lo = window > 0 ? max(0, pos - window + 1) : 0;
+    if (chunk > 0) lo = max(lo, pos - pos % chunk);
+    return lo;
+}
+
+// A sink's term of a softmax denominator: sinks[head] is one more score of that query head (natural units, not
+// scaled) that has no key and no value.  Exponentials are taken as 2^(x - ref) with ref in units of log2.
+__device__ __forceinline__ float sink_term(const float* __restrict__ sinks, int head, float ref) {
+    return sinks ? fast_exp2(sinks[head] * LOG2E - ref) : 0.f;
+}
+
 // Maximum and sum over the four lanes r, r+16, r+32, r+48 that share a q column, for every lane, by the
 // register swaps between the wave's rows of 16 lanes (no trip through LDS as a general lane shuffle makes):
 // v_permlane16_swap exchanges rows 1, 3 of its first operand with rows 0, 2 of its second, v_permlane32_swap
@@ -358,9 +372,10 @@ __host__ __device__ inline int decode_splits(int n_tiles) {
 // out = sum_s w_s acc_s / sum_s w_s l_s over the splits of one (sequence, head), with w_s = 2^(m_s - max m) (the
 // maxima are kept in units of log2; a split without keys has m = -inf and weight 0).  One element: `at(s)` gives
 // split s's (acc, m, l).  Summed in split order with fused multiply-adds, the same wherever it is called from.
+// `beside` is what the denominator holds beside the keys (a sink's term, relative to mx; else 0).
 template <typename At>
-__device__ __forceinline__ float merge_splits(int n_splits, float mx, At at) {
-    float o = 0.f, denom = 0.f;
+__device__ __forceinline__ float merge_splits(int n_splits, float mx, float beside, At at) {
+    float o = 0.f, denom = beside;
     for (int s0 = 0; s0 < n_splits; s0 += 4) {  // four splits' loads in flight at a time
         float acc[4], m[4], l[4];
 #pragma unroll
@@ -430,7 +445,8 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ cu_q,
     const int* __restrict__ kv_len, float* __restrict__ ws_acc, float* __restrict__ ws_ml,
-    bf16_t* __restrict__ out, int n_heads, int n_kv, int ps_log2, float scale, int window, int max_splits, int mode) {
+    bf16_t* __restrict__ out, int n_heads, int n_kv, int ps_log2, float scale, int window, int chunk,
+    const float* __restrict__ sinks, int max_splits, int mode) {
     const bool fold = mode == DEC_FOLD, spread = mode == DEC_SPREAD;
     static_assert(DEC_WAVES == 4, "merge_waves merges four runs");
     extern __shared__ float lds[];  // [runs of the workgroup][group][HD + 2]
@@ -439,7 +455,7 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
     const int hk = blockIdx.x, seq = blockIdx.y;
     const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     const int pos = kv_len[seq] - 1;
-    const int lo_all = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lo_all = first_visible(pos, window, chunk);
     const int t_first = lo_all / TILE, n_tiles = pos / TILE - t_first + 1;
     const int n_splits = min(decode_splits(n_tiles), max_splits);
     // the whole workgroup leaves: the grid is sized for the longest sequence there may be
@@ -508,7 +524,7 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
             float o, mx, lsum;
             merge_waves([&](int w) { return lds + (size_t)(w * group + c) * ROW; }, d, o, mx, lsum);
             if (n_splits == 1) {  // nothing to combine with: this is the result
-                *dst = float_to_bf16(o * (1.f / lsum));
+                *dst = float_to_bf16(o * (1.f / (lsum + sink_term(sinks, hk * group + c, mx))));
                 continue;
             }
             const size_t slot = ((size_t)seq * n_heads + hk * group + c) * max_splits + blockIdx.z;
@@ -521,7 +537,8 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
         }
         float mx_all = -INFINITY;
         for (int run = 0; run < n_runs; ++run) mx_all = fmaxf(mx_all, lds[(size_t)(run * group + c) * ROW + HD]);
-        *dst = float_to_bf16(merge_splits(n_splits, mx_all, [&](int sp, float& a, float& m, float& l) {
+        *dst = float_to_bf16(merge_splits(n_splits, mx_all, sink_term(sinks, hk * group + c, mx_all),
+                                          [&](int sp, float& a, float& m, float& l) {
             merge_waves([&](int w) { return lds + (size_t)((sp * DEC_WAVES + w) * group + c) * ROW; }, d, a, m, l);
         }));
     }
@@ -531,10 +548,11 @@ __global__ __launch_bounds__(DEC_WAVES* SIA_WAVE) void attn_decode_kernel(
 // (ws_acc [..][split][HD], ws_ml [..][split][2]), or with `runs` the states of all runs (ws_acc [..][run][HD + 2]).
 __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
     const float* __restrict__ ws_acc, const float* __restrict__ ws_ml, const int* __restrict__ cu_q,
-    const int* __restrict__ kv_len, bf16_t* __restrict__ out, int n_heads, int max_splits, int window, int runs) {
+    const int* __restrict__ kv_len, bf16_t* __restrict__ out, int n_heads, int max_splits, int window, int chunk,
+    const float* __restrict__ sinks, int runs) {
     const int head = blockIdx.x, seq = blockIdx.y, lane = threadIdx.x;
     const int pos = kv_len[seq] - 1;
-    const int lo_all = window > 0 ? max(0, pos - window + 1) : 0;
+    const int lo_all = first_visible(pos, window, chunk);
     const int n_splits = min(decode_splits(pos / TILE - lo_all / TILE + 1), max_splits);
     bf16_t* dst = out + ((size_t)cu_q[seq] * n_heads + head) * HD;
     if (runs) {
@@ -544,7 +562,8 @@ __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
         for (int run = lane; run < n_splits * DEC_WAVES; run += SIA_WAVE) mx = fmaxf(mx, mine[(size_t)run * ROW + HD]);
         mx = wave_max(mx);
         for (int d = lane; d < HD; d += SIA_WAVE)
-            dst[d] = float_to_bf16(merge_splits(n_splits, mx, [&](int sp, float& acc, float& m, float& l) {
+            dst[d] = float_to_bf16(merge_splits(n_splits, mx, sink_term(sinks, head, mx),
+                                                [&](int sp, float& acc, float& m, float& l) {
                 merge_waves([&](int w) { return mine + (size_t)(sp * DEC_WAVES + w) * ROW; }, d, acc, m, l);
             }));
         return;
@@ -555,7 +574,8 @@ __global__ __launch_bounds__(SIA_WAVE) void attn_decode_combine_kernel(
     for (int s = lane; s < n_splits; s += SIA_WAVE) mx = fmaxf(mx, ws_ml[(base + s) * 2]);
     mx = wave_max(mx);
     for (int d = lane; d < HD; d += SIA_WAVE)
-        dst[d] = float_to_bf16(merge_splits(n_splits, mx, [&](int s, float& acc, float& m, float& l) {
+        dst[d] = float_to_bf16(merge_splits(n_splits, mx, sink_term(sinks, head, mx),
+                                            [&](int s, float& acc, float& m, float& l) {
             acc = ws_acc[(base + s) * HD + d];
             m = ws_ml[(base + s) * 2];
             l = ws_ml[(base + s) * 2 + 1];
@@ -738,7 +758,7 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, int q_row_stride, const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ cu_q,
     const int* __restrict__ kv_len, bf16_t* __restrict__ out, int n_heads, int n_kv, int ps_log2, float scale,
-    int window, int seq_begin, int seq_end) {
+    int window, int chunk, const float* __restrict__ sinks, int seq_begin, int seq_end) {
     constexpr int ROW_WAVES = PF_WAVES / KSPLIT;
     constexpr int ROWS = ROW_WAVES * PF_NQ * 16;
     constexpr int TEAM = PF_WAVES * SIA_WAVE;
@@ -794,7 +814,7 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
         const int qpos = first_pos + row;
         load_q(qf[n], live ? q + (size_t)(q_begin + row) * q_row_stride + head * HD : nullptr, g);
         hi[n] = live ? qpos : 0;
-        lo[n] = live ? (window > 0 ? max(0, qpos - window + 1) : 0) : 1;
+        lo[n] = live ? first_visible(qpos, window, chunk) : 1;
 #pragma unroll
         for (int db = 0; db < DBLOCKS; ++db) acc[n][db] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
@@ -808,9 +828,9 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
         // the workgroup's key range: from the first row's oldest visible key to the last live row's position
         const int blk_rows = min(q_len - tile * ROWS, ROWS);
         const int blk_hi = first_pos + tile * ROWS + blk_rows - 1;
-        const int blk_lo = window > 0 ? max(0, first_pos + tile * ROWS - window + 1) : 0;
+        const int blk_lo = first_visible(first_pos + tile * ROWS, window, chunk);
         const int wave_hi = first_pos + row_last;
-        const int wave_lo = window > 0 ? max(0, first_pos + row0 - window + 1) : 0;
+        const int wave_lo = first_visible(first_pos + row0, window, chunk);
         const int kb_first = (blk_lo / TILE) * TILE, kb_last = (blk_hi / TILE) * TILE;
         constexpr int STEP_KEYS = KTILES * TILE;
         constexpr int AHEAD = PF_NQ == 1 ? 4 : 2;
@@ -897,7 +917,7 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
         static_assert(PF_USE_LDS || KSPLIT == 1, "the split shape stages its tiles through LDS");
         if (wave_live) {
             const int range_hi = first_pos + row_last;
-            const int range_lo = window > 0 ? max(0, first_pos + row0 - window + 1) : 0;
+            const int range_lo = first_visible(first_pos + row0, window, chunk);
             attend_range<PF_NQ>(qf, kp, vp, table, table_width, ps_log2, n_kv, hk, range_lo, range_hi, lo, hi, scale,
                                 sm, acc);
         }
@@ -930,6 +950,7 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
             const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
             const float w_mine = fast_exp2(sm.m[n] - m_use), w_other = fast_exp2(m_other - m_use);
             sm.l[n] = sm.l[n] * w_mine + b[1] * w_other;
+            sm.m[n] = m_use;
 #pragma unroll
             for (int db = 0; db < DBLOCKS; ++db)
 #pragma unroll
@@ -942,7 +963,7 @@ __global__ __launch_bounds__(PF_WAVES* SIA_WAVE) void attn_prefill_kernel(
     for (int n = 0; n < PF_NQ; ++n) {
         const int row = row0 + n * 16 + r;
         if (row >= q_len) continue;
-        const float inv = 1.f / sm.l[n];
+        const float inv = 1.f / (sm.l[n] + sink_term(sinks, head, sm.m[n]));
         bf16_t* dst = out + ((size_t)(q_begin + row) * n_heads + head) * HD;
 #pragma unroll
         for (int db = 0; db < DBLOCKS; ++db) {
@@ -978,7 +999,8 @@ static int log2_exact(int v) {
 SIA_EXPORT int sia_attn_mfma_head_dim() { return HD; }
 
 // Most workgroups that share one (sequence, kv head) when no sequence of the step holds more than kv_bound keys
-// (with a window: sees more than the window): what the caller sizes the workspaces and this library its grid by.
+// (with a window: sees more than the window; for queries that see a block of positions `window` is the block's
+// size): what the caller sizes the workspaces and this library its grid by.
 SIA_EXPORT int sia_attn_decode_max_splits(int kv_bound, int window) {
     if (kv_bound <= 0) return 1;
     // the visible keys of a sequence of length n span at most this many tiles (a window need not start on a tile)
@@ -1019,10 +1041,13 @@ SIA_EXPORT long long sia_attn_decode_workspace(int n_seqs, int n_heads, int n_kv
 // Sequences 0 .. n_seqs-1 of the step, each with exactly one new token, which is row s of q (cu_q[s] = s), and
 // none longer than kv_bound.  max_splits = sia_attn_decode_max_splits(kv_bound, window); ws_acc and ws_ml hold
 // sia_attn_decode_workspace(.., 0) and (.., 1) floats (neither is read before it is written).
-SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
-                               const int* block_table, int table_width, const int* cu_q, const int* kv_len,
-                               void* out, float* ws_acc, float* ws_ml, int n_seqs, int n_heads, int n_kv,
-                               int page_size, float scale, int window, int max_splits, hipStream_t stream) {
+// chunk > 0: a query sees only its own block of chunk positions (max_splits then from min(window, chunk), whichever
+// are given); sinks: one float per query head that joins its softmax's denominator, or null.
+SIA_EXPORT int sia_attn_decode_ex(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
+                                  const int* block_table, int table_width, const int* cu_q, const int* kv_len,
+                                  void* out, float* ws_acc, float* ws_ml, int n_seqs, int n_heads, int n_kv,
+                                  int page_size, float scale, int window, int chunk, const float* sinks,
+                                  int max_splits, hipStream_t stream) {
     if (n_seqs <= 0) return 0;
     const int ps_log2 = log2_exact(page_size);
     const int n_splits = max_splits;
@@ -1054,11 +1079,20 @@ SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pa
     hipLaunchKernelGGL(attn_decode_kernel, grid, dim3((mode == DEC_SPREAD ? 1 : DEC_WAVES) * SIA_WAVE),
                        mode == DEC_SPREAD ? 0 : lds_bytes, stream, (const bf16_t*)q, q_row_stride,
                        (const bf16_t*)k_pages, (const bf16_t*)v_pages, block_table, table_width, cu_q, kv_len, ws_acc,
-                       ws_ml, (bf16_t*)out, n_heads, n_kv, ps_log2, scale, window, n_splits, (int)mode);
+                       ws_ml, (bf16_t*)out, n_heads, n_kv, ps_log2, scale, window, chunk, sinks, n_splits, (int)mode);
     if (mode == DEC_SPREAD || (mode == DEC_PLAIN && n_splits > 1))
         hipLaunchKernelGGL(attn_decode_combine_kernel, dim3(n_heads, n_seqs), dim3(SIA_WAVE), 0, stream, ws_acc,
-                           ws_ml, cu_q, kv_len, (bf16_t*)out, n_heads, n_splits, window, mode == DEC_SPREAD ? 1 : 0);
+                           ws_ml, cu_q, kv_len, (bf16_t*)out, n_heads, n_splits, window, chunk, sinks,
+                           mode == DEC_SPREAD ? 1 : 0);
     return SIA_LAUNCH_CHECK();
+}
+
+SIA_EXPORT int sia_attn_decode(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
+                               const int* block_table, int table_width, const int* cu_q, const int* kv_len,
+                               void* out, float* ws_acc, float* ws_ml, int n_seqs, int n_heads, int n_kv,
+                               int page_size, float scale, int window, int max_splits, hipStream_t stream) {
+    return sia_attn_decode_ex(q, q_row_stride, k_pages, v_pages, block_table, table_width, cu_q, kv_len, out, ws_acc,
+                              ws_ml, n_seqs, n_heads, n_kv, page_size, scale, window, 0, nullptr, max_splits, stream);
 }
 
 // Sequences seq_begin .. seq_end-1 of the step.  n_tiles = sum over them of ceil(q_len / sia_attn_prefill_rows()),
@@ -1072,7 +1106,7 @@ template <int NQ, int WAVES, int KSPLIT, int KTILES = KSPLIT>
 static int launch_prefill(int tiles, const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
                           const int* block_table, int table_width, const int* cu_q, const int* kv_len, void* out,
                           int seq_begin, int seq_end, int n_heads, int n_kv, int ps_log2, float scale, int window,
-                          hipStream_t stream) {
+                          int chunk, const float* sinks, hipStream_t stream) {
     constexpr int TILE_ELEMS = TILE * K_STRIDE + HD * V_STRIDE;
     size_t lds_bytes = PF_USE_LDS ? (size_t)2 * KTILES * TILE_ELEMS * sizeof(bf16_t) : 0;
     if (KSPLIT == 2) {
@@ -1087,7 +1121,7 @@ static int launch_prefill(int tiles, const void* q, int q_row_stride, const void
     hipLaunchKernelGGL((attn_prefill_kernel<NQ, WAVES, KSPLIT, KTILES>), dim3(tiles, n_heads), dim3(WAVES * SIA_WAVE),
                        lds_bytes, stream, (const bf16_t*)q, q_row_stride, (const bf16_t*)k_pages,
                        (const bf16_t*)v_pages, block_table, table_width, cu_q, kv_len, (bf16_t*)out, n_heads, n_kv,
-                       ps_log2, scale, window, seq_begin, seq_end);
+                       ps_log2, scale, window, chunk, sinks, seq_begin, seq_end);
     return SIA_LAUNCH_CHECK();
 }
 
@@ -1123,17 +1157,17 @@ static PrefillShape prefill_shape(int n_tiles, int n_tiles_split, int n_tiles_lo
     return PF_WIDE;
 }
 
-SIA_EXPORT int sia_attn_prefill(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
-                                const int* block_table, int table_width, const int* cu_q, const int* kv_len,
-                                void* out, int seq_begin, int seq_end, int n_tiles, int n_tiles_split, int n_tiles_long,
-                                int q_bound, int kv_bound, int n_heads, int n_kv, int page_size, float scale, int window,
-                                hipStream_t stream) {
+SIA_EXPORT int sia_attn_prefill_ex(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
+                                   const int* block_table, int table_width, const int* cu_q, const int* kv_len,
+                                   void* out, int seq_begin, int seq_end, int n_tiles, int n_tiles_split,
+                                   int n_tiles_long, int q_bound, int kv_bound, int n_heads, int n_kv, int page_size,
+                                   float scale, int window, int chunk, const float* sinks, hipStream_t stream) {
     if (seq_end <= seq_begin || n_tiles <= 0) return 0;
     const int ps_log2 = log2_exact(page_size);
     if (ps_log2 < 3 || n_kv <= 0 || n_heads % n_kv || n_heads > 65535 || q_row_stride % 8 || table_width <= 0)
         return SIA_BAD_ARGUMENT;
 #define ARGS q, q_row_stride, k_pages, v_pages, block_table, table_width, cu_q, kv_len, out, seq_begin, seq_end, \
-             n_heads, n_kv, ps_log2, scale, window, stream
+             n_heads, n_kv, ps_log2, scale, window, chunk, sinks, stream
     if constexpr (HD > 128 || !PF_USE_LDS) {
         return HD > 128 ? launch_prefill<1, PF_ROWS / 16, 1>(n_tiles, ARGS) : launch_prefill<2, PF_ROWS / 32, 1>(n_tiles, ARGS);
     } else {
@@ -1145,4 +1179,14 @@ SIA_EXPORT int sia_attn_prefill(const void* q, int q_row_stride, const void* k_p
         }
     }
 #undef ARGS
+}
+
+SIA_EXPORT int sia_attn_prefill(const void* q, int q_row_stride, const void* k_pages, const void* v_pages,
+                                const int* block_table, int table_width, const int* cu_q, const int* kv_len,
+                                void* out, int seq_begin, int seq_end, int n_tiles, int n_tiles_split, int n_tiles_long,
+                                int q_bound, int kv_bound, int n_heads, int n_kv, int page_size, float scale, int window,
+                                hipStream_t stream) {
+    return sia_attn_prefill_ex(q, q_row_stride, k_pages, v_pages, block_table, table_width, cu_q, kv_len, out, seq_begin,
+                               seq_end, n_tiles, n_tiles_split, n_tiles_long, q_bound, kv_bound, n_heads, n_kv, page_size,
+                               scale, window, 0, nullptr, stream);
 }

@@ -32,6 +32,17 @@ template <typename T> __device__ __forceinline__ T from_float(float x);
 template <> __device__ __forceinline__ float from_float<float>(float x) { return x; }
 template <> __device__ __forceinline__ bf16_t from_float<bf16_t>(float x) { return float_to_bf16(x); }
 
+// Activations without a gate, in float:  SIA_RELU2: max(z, 0)^2;  SIA_GELU_TANH: 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
+enum SiaActivation { SIA_RELU2 = 0, SIA_GELU_TANH = 1 };
+
+__device__ __forceinline__ float activate(float z, int kind) {
+    if (kind == SIA_RELU2) {
+        const float r = fmaxf(z, 0.f);
+        return r * r;
+    }
+    return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
 // Eight consecutive elements of a row as one register value: 32 bytes of float or 16 of bfloat16.
 template <typename T> struct Vec8;
 template <> struct Vec8<float> {

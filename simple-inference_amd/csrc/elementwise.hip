@@ -1,4 +1,5 @@
-// Embedding gather, residual add + RMS norm, SwiGLU activation.
+// Embedding gather, residual add + RMS norm, RMS norm of a sublayer's output + residual add, SwiGLU and plain
+// activations.
 //
 // These are bound by memory traffic or by launch latency.  The residual stream is float
 // in both modes; rows are handled by one workgroup each, with vector accesses where the
@@ -6,25 +7,25 @@
 #include "common.h"
 
 // ---------------------------------------------------------------------------------------
-// Embedding: out[n, :] = float(table[ids[n], :])          (reference: ops/embedding.py:57-60)
+// Embedding: out[n, :] = float(table[ids[n], :]) * scale   (reference: ops/embedding.py:57-60; scale 1 there)
 // ---------------------------------------------------------------------------------------
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table,
-                             float* __restrict__ out, int hidden) {
+                             float* __restrict__ out, int hidden, float scale) {
     const int n = blockIdx.x;
     const T* src = table + (size_t)ids[n] * hidden;
     float* dst = out + (size_t)n * hidden;
-    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_float(src[i]) * scale;
 }
 
 SIA_EXPORT int sia_embed(const int* ids, const void* table, float* out, int n_tokens, int hidden,
-                         int table_dtype, hipStream_t stream) {
+                         int table_dtype, float scale, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     dim3 grid(n_tokens), block(256);
     if (table_dtype == SIA_F32)
-        hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, ids, (const float*)table, out, hidden);
+        hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, ids, (const float*)table, out, hidden, scale);
     else if (table_dtype == SIA_BF16)
-        hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, ids, (const bf16_t*)table, out, hidden);
+        hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, ids, (const bf16_t*)table, out, hidden, scale);
     else
         return SIA_BAD_ARGUMENT;
     return SIA_LAUNCH_CHECK();
@@ -135,6 +136,128 @@ SIA_EXPORT int sia_add_rmsnorm(float* residual, const void* delta, const float* 
     else
         hipLaunchKernelGGL(add_rmsnorm_kernel<bf16_t>, grid, block, 0, stream, residual, (const bf16_t*)delta,
                            weight, (bf16_t*)out, rows, hidden, eps);
+    return SIA_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
+// RMS norm of a sublayer's output, added into the residual:
+//
+//   residual[row] += y[row] * rsqrt(mean(y[row]^2) + eps) * w         (all float)
+//   lowered[row]   = the new residual[row], rounded to T               (if lowered is given)
+//
+// for layers whose norm sits behind the sublayer and whose sublayers read the residual itself.  One workgroup a
+// row; the sum of squares is reduced in a fixed order that depends on the row length only.
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void norm_add_kernel(float* __restrict__ residual, const T* __restrict__ y,
+                                const float* __restrict__ weight, T* __restrict__ lowered, int hidden, float eps) {
+    __shared__ float scratch[16];
+    const size_t base = (size_t)blockIdx.x * hidden;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float v = to_float(y[base + i]);
+        ss += v * v;
+    }
+    ss = block_sum(ss, scratch);
+    const float inv = rsqrtf(ss / (float)hidden + eps);
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+        const float x = residual[base + i] + to_float(y[base + i]) * inv * weight[i];
+        residual[base + i] = x;
+        if (lowered) lowered[base + i] = from_float<T>(x);
+    }
+}
+
+// The same for rows that one workgroup holds in registers (hidden % 8 == 0, hidden <= 8 * 1024): 8 consecutive
+// elements a thread, every input read once, all loads issued before the first is used.
+template <typename T>
+__global__ void norm_add_row_kernel(float* __restrict__ residual, const T* __restrict__ y,
+                                    const float* __restrict__ weight, T* __restrict__ lowered, int hidden, float eps) {
+    __shared__ float scratch[16];
+    const size_t base = (size_t)blockIdx.x * hidden;
+    const int i0 = threadIdx.x * 8;
+    const bool live = i0 < hidden;
+    float x[8], w[8], v[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (live) {
+        Vec8<float> vr, vw;
+        Vec8<T> vy;
+        vr.load(residual + base + i0);
+        vw.load(weight + i0);
+        vy.load(y + base + i0);
+        vr.get(x);
+        vw.get(w);
+        vy.get(v);
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ss += v[i] * v[i];
+    ss = block_sum(ss, scratch);
+    if (live) {
+        const float inv = rsqrtf(ss / (float)hidden + eps);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] += v[i] * inv * w[i];
+        Vec8<float> vr;
+        vr.set(x);
+        vr.store(residual + base + i0);
+        if (lowered) {
+            Vec8<T> vo;
+            vo.set(x);
+            vo.store(lowered + base + i0);
+        }
+    }
+}
+
+SIA_EXPORT int sia_norm_add(float* residual, const void* y, const float* weight, void* lowered, int n_rows,
+                            int hidden, float eps, int dtype, hipStream_t stream) {
+    if (n_rows <= 0) return 0;
+    if ((dtype != SIA_F32 && dtype != SIA_BF16) || hidden <= 0 || !residual || !y || !weight) return SIA_BAD_ARGUMENT;
+    dim3 grid(n_rows);
+    const bool row = hidden % 8 == 0 && hidden <= 8 * 1024;
+    dim3 block(row ? ((hidden / 8 + SIA_WAVE - 1) / SIA_WAVE) * SIA_WAVE : (hidden >= 2048 ? 512 : 256));
+#define LAUNCH(KERNEL, T)                                                                                         \
+    hipLaunchKernelGGL(KERNEL<T>, grid, block, 0, stream, residual, (const T*)y, weight, (T*)lowered, hidden, eps)
+    if (row) {
+        if (dtype == SIA_F32) LAUNCH(norm_add_row_kernel, float);
+        else LAUNCH(norm_add_row_kernel, bf16_t);
+    } else {
+        if (dtype == SIA_F32) LAUNCH(norm_add_kernel, float);
+        else LAUNCH(norm_add_kernel, bf16_t);
+    }
+#undef LAUNCH
+    return SIA_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------
+// Plain activations, in float on the stored value, rounded once:
+//   SIA_RELU2:      max(z, 0)^2
+//   SIA_GELU_TANH:  0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ void activation_kernel(const T* __restrict__ in, T* __restrict__ out, size_t n, int kind) {
+    const size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    if (i >= n) return;
+    if (i + 8 <= n) {
+        Vec8<T> v;
+        float z[8];
+        v.load(in + i);
+        v.get(z);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) z[j] = activate(z[j], kind);
+        v.set(z);
+        v.store(out + i);
+    } else {
+        for (size_t j = i; j < n; ++j) out[j] = from_float<T>(activate(to_float(in[j]), kind));
+    }
+}
+
+// Eight elements a thread; the last thread takes what is left one by one.
+SIA_EXPORT int sia_activation(const void* in, void* out, long long n, int kind, int dtype, hipStream_t stream) {
+    if (n <= 0) return 0;
+    if ((dtype != SIA_F32 && dtype != SIA_BF16) || (kind != SIA_RELU2 && kind != SIA_GELU_TANH)) return SIA_BAD_ARGUMENT;
+    dim3 block(256), grid((unsigned)(((n + 7) / 8 + 255) / 256));
+    if (dtype == SIA_F32)
+        hipLaunchKernelGGL(activation_kernel<float>, grid, block, 0, stream, (const float*)in, (float*)out, (size_t)n, kind);
+    else
+        hipLaunchKernelGGL(activation_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)in, (bf16_t*)out, (size_t)n, kind);
     return SIA_LAUNCH_CHECK();
 }
 

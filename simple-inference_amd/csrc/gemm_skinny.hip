@@ -38,7 +38,7 @@ __device__ __forceinline__ bf16x8 ld8(const bf16_t* p) {
     return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p));
 }
 
-enum SkinnyEpilogue { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_ROPE = 2, EPI_RESIDUAL = 3 };
+enum SkinnyEpilogue { EPI_STORE = 0, EPI_SWIGLU = 1, EPI_ROPE = 2, EPI_RESIDUAL = 3, EPI_ACT = 4 };
 
 // What the q/k/v product needs to rotate its result and to put keys and values into the cache pages.
 struct RopeOut {
@@ -71,10 +71,12 @@ struct Epilogue {
     RopeOut rope;
     ResidualOut res;
     RowScale scale;
+    int activation;   // EPI_ACT: which (SiaActivation)
 };
 
 // RB: blocks of bh rows of W per workgroup; WAVES: 8 or 16 waves that split K.
 //   EPI_STORE:   row block rb holds bh rows of W and gives as many columns of Y (TOut)
+//   EPI_ACT:     as EPI_STORE, with an activation without a gate applied to the float sums, rounded once
 //   EPI_SWIGLU:  W = [gate; up] of N rows each; the first RB / 2 row blocks are gate rows, the others the up rows of
 //                the same columns: Y = silu(gate) * up, in float, rounded once
 //   EPI_ROPE:    RB = 2, W = [q heads | k heads | v heads] of head_dim rows each; a workgroup owns 16 columns of
@@ -305,6 +307,8 @@ __global__ __launch_bounds__(WAVES* SIA_WAVE) void gemm_skinny_kernel(const bf16
             gate *= rs;
             up *= rs;
             *y = from_float<TOut>(gate / (1.f + expf(-gate)) * up);
+        } else if (EPI == EPI_ACT) {
+            *y = from_float<TOut>(activate(total(j, m, n) * rs, ep.activation));
         } else {
             *y = from_float<TOut>(total(j, m, n) * rs);
         }
@@ -384,6 +388,17 @@ SIA_EXPORT int sia_gemm_skinny(const void* X, const void* W, void* Y, int M, int
         launch_skinny<float, EPI_STORE>((const bf16_t*)X, (const bf16_t*)W, (float*)Y, M, N, K, Epilogue{}, stream);
     else
         launch_skinny<bf16_t, EPI_STORE>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, N, K, Epilogue{}, stream);
+    return SIA_LAUNCH_CHECK();
+}
+
+// Y[M, N] = act(X W^T) in bfloat16, act one of SiaActivation.  Needs M <= 16, K % 64 == 0.
+SIA_EXPORT int sia_gemm_skinny_act(const void* X, const void* W, void* Y, int M, int N, int K, int activation,
+                                   hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K % 64 || K <= 0 || (activation != SIA_RELU2 && activation != SIA_GELU_TANH)) return SIA_BAD_ARGUMENT;
+    Epilogue ep{};
+    ep.activation = activation;
+    launch_skinny<bf16_t, EPI_ACT>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)Y, M, N, K, ep, stream);
     return SIA_LAUNCH_CHECK();
 }
 

@@ -22,18 +22,26 @@ import torch
 from . import build
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
+_ACTIVATIONS = {"relu2": 0, "gelu_tanh": 1}   # ``SiaActivation`` of csrc/common.h
 
 _c_int, _c_float, _c_ptr, _c_ll = ctypes.c_int, ctypes.c_float, ctypes.c_void_p, ctypes.c_longlong
 
 _SIGNATURES = {
-    "sia_embed": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_embed": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_ptr],
+    "sia_norm_add": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "sia_activation": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_ptr],
+    "sia_qk_prepare": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
+                       _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_qk_prepare_max_head_dim": [],
+    "sia_gemm_skinny_act": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_add_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "sia_swiglu": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "sia_cast": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_ptr],
     "sia_rope_kv_write": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
                           _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_attention_generic": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
-                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
+                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr, _c_int,
+                              _c_ptr],
     "sia_attention_max_head_dim": [],
     "sia_gemm_generic": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_prenorm_block": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_ptr],
@@ -63,6 +71,11 @@ _ATTN_SIGNATURES = {
     "sia_attn_prefill": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
                          _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int,
                          _c_ptr],
+    "sia_attn_decode_ex": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                           _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr, _c_int, _c_ptr],
+    "sia_attn_prefill_ex": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                            _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float,
+                            _c_int, _c_int, _c_ptr, _c_ptr],
     "sia_attn_decode_max_splits": [_c_int, _c_int],
     "sia_attn_decode_workspace": [_c_int, _c_int, _c_int, _c_int, _c_int],
     "sia_attn_decode_mode": [_c_int, _c_int, _c_int, _c_int],
@@ -277,7 +290,7 @@ class HipKernels:
         self._check(self.core.sia_place_tokens(_ptr(token_ids), _ptr(dst_rows), _ptr(src_tokens), _ptr(src_rows),
                                                dst_rows.numel(), self._stream()), "place_tokens")
 
-    def embed(self, token_ids, table):
+    def embed(self, token_ids, table, scale=1.0):
         self._want(token_ids, "token_ids", torch.int32)
         self._want(table, "embedding table")
         if table.dtype not in _DT or table.dim() != 2:
@@ -285,8 +298,23 @@ class HipKernels:
         n, hidden = token_ids.numel(), table.shape[1]
         out = torch.empty((n, hidden), dtype=torch.float32, device=table.device)
         self._check(self.core.sia_embed(_ptr(token_ids), _ptr(table), _ptr(out), n, hidden, _DT[table.dtype],
-                                        self._stream()), "embed")
+                                        float(scale), self._stream()), "embed")
         return out
+
+    # -- rms norm of a sublayer's output, added into the residual -------------------
+    def norm_add(self, residual, y, weight, eps, out_dtype):
+        """``residual += y * rsqrt(mean(y^2) + eps) * weight`` (float); returns the new residual in ``out_dtype``
+        (the residual itself if that is float32)."""
+        n, hidden = residual.shape
+        self._want(residual, "residual", torch.float32)
+        self._want(weight, "norm weight", torch.float32, (hidden,))
+        if out_dtype not in _DT:
+            raise KernelError(f"norm output dtype {out_dtype} is not float32 or bfloat16")
+        self._want(y, "sublayer output", out_dtype, (n, hidden))
+        lowered = None if out_dtype == torch.float32 else torch.empty((n, hidden), dtype=out_dtype, device=residual.device)
+        self._check(self.core.sia_norm_add(_ptr(residual), _ptr(y), _ptr(weight), _ptr(lowered), n, hidden, float(eps),
+                                           _DT[out_dtype], self._stream()), "norm_add")
+        return residual if lowered is None else lowered
 
     # -- residual add + rms norm ---------------------------------------------
     def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None):
@@ -356,6 +384,35 @@ class HipKernels:
                         "gemm_skinny_swiglu")
             return y
         return self.swiglu(self.linear(x, w_gate_up))
+
+    def activated_linear(self, x, w, activation):
+        """``act(x @ w^T)`` for an activation without a gate (``relu2``, ``gelu_tanh``): one kernel for few rows,
+        else the product and the activation."""
+        if activation not in _ACTIVATIONS:
+            raise KernelError(f"activation {activation!r} is not one of {', '.join(_ACTIVATIONS)}")
+        x = self.finish_rows(x)
+        self._want(x, "linear input")
+        self._want(w, "linear weight")
+        if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+            raise KernelError(f"linear shapes do not fit: x {tuple(x.shape)}, w {tuple(w.shape)}")
+        M, K = x.shape
+        N = w.shape[0]
+        if (self.use_skinny_gemm and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+                and 0 < M <= self._skinny_rows and K % 64 == 0):
+            y = torch.empty((M, N), dtype=torch.bfloat16, device=x.device)
+            self._check(self.core.sia_gemm_skinny_act(_ptr(x), _ptr(w), _ptr(y), M, N, K, _ACTIVATIONS[activation],
+                                                      self._stream()), "gemm_skinny_act")
+            return y
+        return self.activation(self.linear(x, w), activation)
+
+    def activation(self, z, activation):
+        self._want(z, "activation input")
+        if z.dtype not in _DT:
+            raise KernelError(f"activation takes float32 or bfloat16, got {z.dtype}")
+        out = torch.empty_like(z)
+        self._check(self.core.sia_activation(_ptr(z), _ptr(out), z.numel(), _ACTIVATIONS[activation], _DT[z.dtype],
+                                             self._stream()), "activation")
+        return out
 
     # -- a product whose result goes into the residual, and the norm after it ---------
     def pending_linear(self, x, w):
@@ -501,11 +558,21 @@ class HipKernels:
             n, n_heads, n_kv_written, head_dim, rotary_dim, page_size, _DT[qkv.dtype], self._stream()),
             "rope_kv_write")
 
-    def qkv_to_cache(self, x, w_qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache):
+    def qkv_to_cache(self, x, w_qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache,
+                     value_dim=None, bias=None, qk_norm=None):
         """The q/k/v product, the rotation of q and k and the write of k and v into the pages.  Returns the
         ``[tokens, (n_heads + 2 n_kv_written) head_dim]`` matrix whose q columns hold the rotated queries; its
-        k and v columns are not to be read (for few rows one kernel does all three and never writes them)."""
+        k and v columns are not to be read (for few rows one kernel does all three and never writes them).
+
+        ``value_dim``: width of a v head if not ``head_dim``; ``bias``: float ``[row width]``, added to the product;
+        ``qk_norm``: ``(q_gain, k_gain, eps)``, an RMS norm over every q and k head before the rotation.  With any
+        of these the product is followed by one kernel that does all of bias, norm, rotation and cache write."""
         M, K = x.shape
+        if value_dim is not None or bias is not None or qk_norm is not None:
+            qkv = self.linear(x, w_qkv)
+            self.qk_prepare(qkv, n_heads, n_kv_written, head_dim, value_dim or head_dim, rotary_dim, cos, sin, bias,
+                            qk_norm, ctx, cache)
+            return qkv
         if (self.use_skinny_gemm and self.fuse_rope and n_kv_written and x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16
                 and M <= self._skinny_rows and rotary_dim == head_dim and head_dim % 2 == 0 and K % 64 == 0):
             x, partials, n_partials, norm_eps = self._scaled(x)
@@ -535,14 +602,57 @@ class HipKernels:
         self.rope_kv_write(qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache)
         return qkv
 
-    def _check_pages(self, k_pages, v_pages, table, page_size, n_kv, head_dim, dtype, ctx):
+    def qk_prepare(self, qkv, n_heads, n_kv_written, head_dim, value_dim, rotary_dim, cos, sin, bias, qk_norm, ctx,
+                   cache):
+        """Bias, per-head RMS norm of q and k, rotation, and the write of k and v into the pages, on the projected
+        rows ``[q heads | k heads | v heads]`` (q and k heads ``head_dim`` wide, v heads ``value_dim``); q is left in
+        place."""
+        self._want(qkv, "qkv")
+        n, width = qkv.shape
+        if qkv.dtype not in _DT:
+            raise KernelError(f"qkv must be float32 or bfloat16, is {qkv.dtype}")
+        if width != n_heads * head_dim + n_kv_written * (head_dim + value_dim):
+            raise KernelError(f"qkv row of {width} does not hold {n_heads} q heads and {n_kv_written} k heads of "
+                              f"{head_dim} and as many v heads of {value_dim}")
+        if n != ctx.n_tokens:
+            raise KernelError(f"qkv has {n} rows, the step {ctx.n_tokens} tokens")
+        if not 0 < head_dim <= self.core.sia_qk_prepare_max_head_dim():
+            raise KernelError(f"head size {head_dim} is outside what the kernel takes")
+        if rotary_dim:
+            for t, what in ((cos, "cos table"), (sin, "sin table")):
+                self._want(t, what, torch.float32)
+                if t.shape[1] != rotary_dim // 2 or t.shape[0] <= ctx.max_kv_len - 1:
+                    raise KernelError(f"{what} {tuple(t.shape)} does not cover position {ctx.max_kv_len - 1} "
+                                      f"with {rotary_dim // 2} pairs")
+        if bias is not None:
+            self._want(bias, "q/k/v bias", torch.float32, (width,))
+        q_gain = k_gain = None
+        eps = 0.0
+        if qk_norm is not None:
+            q_gain, k_gain, eps = qk_norm
+            self._want(q_gain, "q norm gain", torch.float32, (head_dim,))
+            self._want(k_gain, "k norm gain", torch.float32, (head_dim,))
+        table = k_pages = v_pages = None
+        page_size = 0
+        if n_kv_written:
+            k_pages, v_pages, table, page_size = cache.k_pages, cache.v_pages, cache.block_table, cache.page_size
+            self._check_pages(k_pages, v_pages, table, page_size, n_kv_written, head_dim, qkv.dtype, ctx, value_dim)
+        self._check(self.core.sia_qk_prepare(
+            _ptr(qkv), width, _ptr(bias), _ptr(q_gain), _ptr(k_gain), float(eps),
+            _ptr(cos) if rotary_dim else None, _ptr(sin) if rotary_dim else None, _ptr(ctx.positions),
+            _ptr(ctx.seq_of_token), _ptr(table), table.shape[1] if table is not None else 0, _ptr(k_pages),
+            _ptr(v_pages), n, n_heads, n_kv_written, head_dim, value_dim, rotary_dim, page_size, _DT[qkv.dtype],
+            self._stream()), "qk_prepare")
+
+    def _check_pages(self, k_pages, v_pages, table, page_size, n_kv, head_dim, dtype, ctx, value_dim=None):
+        value_dim = value_dim or head_dim
         self._want(k_pages, "key pages", dtype)
         self._want(v_pages, "value pages", dtype)
         pages = k_pages.shape[0]
         if tuple(k_pages.shape) != (pages, n_kv, page_size, head_dim):
             raise KernelError(f"key pages {tuple(k_pages.shape)} are not [pages, {n_kv}, {page_size}, {head_dim}]")
-        if tuple(v_pages.shape) != (pages, n_kv, head_dim, page_size):
-            raise KernelError(f"value pages {tuple(v_pages.shape)} are not [pages, {n_kv}, {head_dim}, {page_size}]")
+        if tuple(v_pages.shape) != (pages, n_kv, value_dim, page_size):
+            raise KernelError(f"value pages {tuple(v_pages.shape)} are not [pages, {n_kv}, {value_dim}, {page_size}]")
         self._want(table, "block table", torch.int32)
         if table.dim() != 2 or table.shape[0] != ctx.n_seqs or table.shape[1] * page_size < ctx.max_kv_len:
             raise KernelError(f"block table {tuple(table.shape)} does not cover {ctx.n_seqs} sequences of up to "
@@ -560,32 +670,44 @@ class HipKernels:
         if n_heads > 65535:
             raise KernelError(f"{n_heads} query heads exceed the kernels' grids (65,535)")
 
-    def paged_attention(self, qkv, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache):
+    def paged_attention(self, qkv, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache, value_dim=None,
+                        chunk=None, sinks=None):
+        """Attention of the rows' q columns over the pages.  ``chunk``: a query sees only the keys of its own block
+        of that many positions; ``sinks``: float ``[n_heads]``, one more term ``exp(sink_h)`` in every softmax
+        denominator of head h; ``value_dim``: width of the value rows if not ``head_dim`` (the result is
+        ``[tokens, n_heads * value_dim]``)."""
         self._want(qkv, "qkv")
         n, width = qkv.shape
+        value_dim = int(value_dim or head_dim)
         if width < n_heads * head_dim or n != ctx.n_tokens:
             raise KernelError(f"qkv {tuple(qkv.shape)} does not hold {ctx.n_tokens} rows of {n_heads} heads of {head_dim}")
         self._check_pages(cache.k_pages, cache.v_pages, cache.block_table, cache.page_size, n_kv_heads, head_dim,
-                          qkv.dtype, ctx)
-        out = torch.empty((n, n_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+                          qkv.dtype, ctx, value_dim)
+        if sinks is not None:
+            self._want(sinks, "sinks", torch.float32, (n_heads,))
+        if chunk is not None and chunk <= 0:
+            raise KernelError(f"chunk must be positive, got {chunk}")
+        out = torch.empty((n, n_heads * value_dim), dtype=qkv.dtype, device=qkv.device)
         page = cache.page_size
         if (self.use_mfma_attention and qkv.dtype == torch.bfloat16 and head_dim % 16 == 0 and head_dim <= 256
-                and page >= 8 and width % 8 == 0 and scale > 0):
-            self._mfma_attention(qkv, out, n_heads, n_kv_heads, head_dim, scale, int(window or 0), ctx, cache)
+                and value_dim == head_dim and page >= 8 and width % 8 == 0 and scale > 0):
+            self._mfma_attention(qkv, out, n_heads, n_kv_heads, head_dim, scale, int(window or 0), ctx, cache,
+                                 int(chunk or 0), sinks)
             return out
         self._check(self.core.sia_attention_generic(
             _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(cache.block_table),
             cache.block_table.shape[1], _ptr(ctx.seq_of_token), _ptr(ctx.positions), _ptr(out), n, n_heads,
-            n_kv_heads, head_dim, page, float(scale), int(window or 0), _DT[qkv.dtype],
-            self._stream()), "attention_generic")
+            n_kv_heads, head_dim, value_dim, page, float(scale), int(window or 0), int(chunk or 0), _ptr(sinks),
+            _DT[qkv.dtype], self._stream()), "attention_generic")
         return out
 
-    def _attention_plan(self, lib, device, n_heads, n_kv_heads, head_dim, window, ctx):
+    def _attention_plan(self, lib, device, n_heads, n_kv_heads, head_dim, window, ctx, chunk=0):
         """What the attention launches of a step need beside the tensors: the same for every layer with this
         geometry, so it is worked out once per step and kept with the step's context (workspaces included: a step's
         layers run one after the other)."""
-        key = (n_heads, n_kv_heads, head_dim, window)
+        key = (n_heads, n_kv_heads, head_dim, window, chunk)
         plans = getattr(ctx, "attention_plans", None)
+        span = min(b for b in (window, chunk) if b > 0) if (window > 0 or chunk > 0) else 0   # most keys a query sees
         if plans is not None and key in plans:
             return plans[key]
         group = n_heads // n_kv_heads
@@ -594,7 +716,7 @@ class HipKernels:
         if n_dec:
             # How many workgroups share a (sequence, kv head) is the kernel's decision, from that sequence's own
             # length; the step's longest possible sequence only sizes the grid and the workspaces.
-            max_splits = lib.sia_attn_decode_max_splits(int(ctx.kv_bound or ctx.max_kv_len), window)
+            max_splits = lib.sia_attn_decode_max_splits(int(ctx.kv_bound or ctx.max_kv_len), span)
             ws_acc, ws_ml = (
                 torch.empty((floats,), dtype=torch.float32, device=device) if floats else None
                 for floats in (lib.sia_attn_decode_workspace(n_dec, n_heads, n_kv_heads, max_splits, which)
@@ -616,24 +738,24 @@ class HipKernels:
         plans[key] = plan
         return plan
 
-    def _mfma_attention(self, qkv, out, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache):
+    def _mfma_attention(self, qkv, out, n_heads, n_kv_heads, head_dim, scale, window, ctx, cache, chunk=0, sinks=None):
         lib = self._attn_lib(head_dim)
         width = qkv.shape[1]
         table = cache.block_table
         n_dec, max_splits, ws_acc, ws_ml, (n_tiles, n_tiles_split, n_tiles_long, q_bound, kv_bound) = \
-            self._attention_plan(lib, qkv.device, n_heads, n_kv_heads, head_dim, window, ctx)
+            self._attention_plan(lib, qkv.device, n_heads, n_kv_heads, head_dim, window, ctx, chunk)
         if n_dec:
-            self._check(lib.sia_attn_decode(
+            self._check(lib.sia_attn_decode_ex(
                 _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
                 _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), _ptr(ws_acc), _ptr(ws_ml), n_dec, n_heads,
-                n_kv_heads, cache.page_size, float(scale), window, max_splits, self._stream()),
+                n_kv_heads, cache.page_size, float(scale), window, chunk, _ptr(sinks), max_splits, self._stream()),
                 "attn_decode")
         if n_dec < ctx.n_seqs:
-            self._check(lib.sia_attn_prefill(
+            self._check(lib.sia_attn_prefill_ex(
                 _ptr(qkv), width, _ptr(cache.k_pages), _ptr(cache.v_pages), _ptr(table), table.shape[1],
                 _ptr(ctx.cu_q), _ptr(ctx.kv_len), _ptr(out), n_dec, ctx.n_seqs, n_tiles, n_tiles_split, n_tiles_long,
-                q_bound, kv_bound, n_heads, n_kv_heads, cache.page_size, float(scale), window, self._stream()),
-                "attn_prefill")
+                q_bound, kv_bound, n_heads, n_kv_heads, cache.page_size, float(scale), window, chunk, _ptr(sinks),
+                self._stream()), "attn_prefill")
 
     # -- a whole block in one call -------------------------------------------------
     def _library_can(self, M, N, K) -> bool:

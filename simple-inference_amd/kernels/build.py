@@ -39,7 +39,7 @@ HIPCC_FLAGS = [
 # name -> sources.  "core" is everything a model needs in either dtype; further libraries
 # are specialisations compiled for the sizes a model has (see ``specialised``).
 LIBRARIES: Dict[str, Sequence[str]] = {
-    "core": ("elementwise.hip", "rope_cache.hip", "attention_generic.hip", "gemm_generic.hip", "gemm_skinny.hip",
+    "core": ("elementwise.hip", "rope_cache.hip", "qk_prepare.hip", "attention_generic.hip", "gemm_generic.hip", "gemm_skinny.hip",
              "sampling.hip", "bandwidth.hip", "block.hip"),
     # the vendor's BLAS library called directly (the products of steps of many tokens); optional: without it those
     # products go through torch
