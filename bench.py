@@ -20,6 +20,11 @@ prompts cut into portions of 512; ``shared-prefix``: 64 requests at the 8B shape
 1,024-token prefix, 256 tokens of their own and 256 decoded tokens each, with and without
 prefix reuse.  They print one JSON line of their own kind.
 
+``--workload feduzen`` measures the Feduzen design beside the Llama model at equal layer sizes (``--shapes``: the
+1B, 3B and 8B widths, head counts and feed-forward sizes; ``--layers`` layers of each, default 8; seeded random
+weights): decode at batch 8 and 1 over 2,048-token contexts and the prefill of 2,048 tokens, each with its
+fraction of the HBM or matrix-core roofline, in one JSON line of its own kind.
+
 The engine runs on one GPU; asked for more it says so and exits with 2.
 """
 
@@ -71,7 +76,9 @@ def parse_args(argv=None):
     ap.add_argument("--temperature", type=float, default=0.0, help="sampling of the decode measurement (0: greedy)")
     ap.add_argument("--top-k", type=int, default=0)
     ap.add_argument("--top-p", type=float, default=1.0)
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "shared-prefix"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "shared-prefix", "feduzen"])
+    ap.add_argument("--shapes", default="1b,3b,8b", help="--workload feduzen: which layer sizes, comma separated")
+    ap.add_argument("--models", default="feduzen,llama", help="--workload feduzen: which of the two models to run")
     ap.add_argument("--max-running", type=int, default=64, help="request slots of the stream workloads")
     return ap.parse_args(argv)
 
@@ -322,6 +329,77 @@ def stream_workload(args):
     return 0
 
 
+FEDUZEN_SHAPES = {   # name -> the Llama preset whose layer sizes both models take
+    "1b": "llama-3.2-1b", "3b": "llama-3.2-3b", "8b": "llama-3.1-8b",
+}
+
+
+def feduzen_config_like(llama_cfg, layers, block=4096):
+    """A Feduzen config.json with the widths, head counts and feed-forward size of a Llama one: full rotation with
+    the same base, the usual score scale, a block mask wider than the measured contexts (every key is seen, as in
+    the Llama model: the kernels do equal work)."""
+    dim = llama_cfg["head_dim"]
+    mixer = {"dim": dim, "vdim": dim, "heads": llama_cfg["num_attention_heads"],
+             "kv_heads": llama_cfg["num_key_value_heads"], "scale": dim ** -0.5, "mask": {"size": block},
+             "rot": {"dims": dim, "base": llama_cfg["rope_theta"],
+                     "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    layer = {"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": llama_cfg["intermediate_size"]}}
+    return {"architecture": "Feduzen", "vocab": llama_cfg["vocab_size"], "width": llama_cfg["hidden_size"],
+            "embedding": {"scale": 1.0}, "norm": {"eps": llama_cfg["rms_norm_eps"]},
+            "layers": [json.loads(json.dumps(layer)) for _ in range(layers)]}
+
+
+def feduzen_workload(args):
+    """Decode and prefill of the Feduzen design beside the Llama model at equal layer sizes."""
+    from simple_inference_amd import Engine, EngineConfig, preset
+
+    layers = args.layers or 8
+    el = 2 if args.dtype == "bfloat16" else 4
+    dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
+    context, T = args.context, args.prefill_tokens
+    total_len = max(context + args.warmup + args.steps + decode_allowance(max(2048, T), 8, context), T + 2)
+    out = {}
+    for shape in [x for x in args.shapes.split(",") if x]:
+        llama = preset(FEDUZEN_SHAPES[shape])
+        llama["num_hidden_layers"] = layers
+        H, I, V = llama["hidden_size"], llama["intermediate_size"], llama["vocab_size"]
+        q, kv = llama["num_attention_heads"] * llama["head_dim"], llama["num_key_value_heads"] * llama["head_dim"]
+        attn_w = H * (q + 2 * kv) + q * H
+        kv_bytes = 2 * layers * kv * el
+        for model, cfg, ff_w, head_w in (("feduzen", feduzen_config_like(llama, layers), 2 * H * I, V * H),
+                                         ("llama", llama, 3 * H * I, V * H)):
+            if model not in args.models.split(","):
+                continue
+            ecfg = EngineConfig(max_running=8, max_seq_len=max(4096, -(-total_len // 1024) * 1024), dtype=args.dtype,
+                                chunk_tokens=max(2048, T), eos_id=-1, use_graphs=not args.no_graphs, device="cuda:0")
+            ecfg.num_kv_blocks = 8 * (-(-total_len // ecfg.block_size)) + 8
+            engine = Engine.from_random(cfg, seed=args.seed, engine_cfg=ecfg, std=0.02, generate_on_device=True)
+            layer_w = layers * (attn_w + ff_w)
+            row = {}
+            for batch in (8, 1):
+                dt, ctx = measure_decode(engine, batch, context, args.steps, args.warmup, args.seed)
+                gbs = ((layer_w + head_w) * el + batch * ctx * kv_bytes) / dt / 1e9
+                row[f"decode_b{batch}"] = {"tok_s": round(batch / dt, 1), "ms_per_step": round(dt * 1e3, 4),
+                                           "hbm_frac": round(gbs / PEAK_HBM_GBS, 4)}
+            if not args.no_prefill:
+                sec, best = measure_prefill(engine, T)
+                flops = 2 * layer_w * T + 2 * head_w + layers * 4 * q * T * (T + 1) / 2
+                row["prefill"] = {"tok_s": round(T / sec, 1), "ms": round(sec * 1e3, 3), "best_ms": round(best * 1e3, 3),
+                                  "matrix_frac": round(flops / sec / PEAK_FLOPS[dt_name], 4)}
+            out.setdefault(shape, {})[model] = row
+            del engine
+            torch.cuda.empty_cache()
+    line = {"metric": "Feduzen beside Llama at equal layer sizes: decode tok/s (batch 8, 1) and prefill tok/s",
+            "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": dt_name,
+            "data": "synthetic (seeded random weights and uniform-random token ids)",
+            "config": {"layers": layers, "context": context, "prefill_tokens": T, "shapes": FEDUZEN_SHAPES,
+                       "feduzen": "full rotation, q/k norm, biases, sinks, a block mask wider than the context, "
+                                  "dense relu^2 feed-forward (two matrices where the gated one has three)"},
+            "shapes": out}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def further_points(args, pts, config, layer_w, head_w, el):
     """What the headline leaves out, at sizes a server meets: the same model with contexts of 8,192 and 32,768 tokens
     and a prompt of 8,192 (an engine of its own with a context limit of 33,792), and the two request streams of the
@@ -388,6 +466,8 @@ def main(argv=None):
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
         return 1
+    if args.workload == "feduzen":
+        return feduzen_workload(args)
     if args.workload != "decode":
         return stream_workload(args)
     points = [int(p) for p in args.points.split(",") if p]

@@ -16,12 +16,60 @@
 // Page layout:  keys   [page][kv_head][offset][head_dim]
 //               values [page][kv_head][value_dim][offset]      (positions innermost)
 //
-// One workgroup a token, one wave a head at a time (the workgroup's waves take the heads in turns), a lane the
-// elements lane, lane + 64, ...
+// A wave takes one q or k head of one token: a lane holds the elements lane, lane + 64, ... of the head, the sum
+// of squares is a butterfly over the wave, and the rotation's partner of an element comes from the lane that holds
+// it by a lane exchange; waves never wait for one another.  A workgroup is four such waves (grid: tokens x groups
+// of four heads), and one more workgroup per token writes the values.  Values lie in a page with positions
+// innermost: where 8 or 16 consecutive tokens of a sequence fill an aligned run of a page, their workgroups share
+// the (head, dim) rows and each writes all the run's positions of its rows at once (16 or 32 contiguous bytes in
+// bfloat16) instead of one element per token and row.
 #include "common.h"
 
 #define QKP_MAX_HEAD_DIM 256
 #define QKP_WAVES 4
+#define QKP_PER_LANE (QKP_MAX_HEAD_DIM / SIA_WAVE)
+
+template <typename T>
+__device__ __forceinline__ void write_values(const T* __restrict__ qkv, int row_stride, const float* __restrict__ bias,
+                                             const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                                             T* __restrict__ v_pages, int n, int n_tokens, int page, int off, int pos,
+                                             int v_first, int rows, int page_size, int v_group) {
+    const T* x = qkv + (size_t)n * row_stride + v_first;
+    const float* b = bias ? bias + v_first : nullptr;
+    bool whole = false;
+    int place = 0, first = n;
+    if (v_group > 0) {
+        const int seq = seq_of_token[n];
+        place = off % v_group;
+        first = n - place;
+        whole = first >= 0 && first + v_group <= n_tokens && seq_of_token[first] == seq &&
+                seq_of_token[first + v_group - 1] == seq && positions[first] == pos - place &&
+                positions[first + v_group - 1] == pos - place + v_group - 1;
+    }
+    if (!whole) {  // an incomplete run: every token writes its own values
+        for (int i = threadIdx.x; i < rows; i += blockDim.x) {
+            float v = to_float(x[i]);
+            if (b) v += b[i];
+            v_pages[((size_t)page * rows + i) * page_size + off] = from_float<T>(v);
+        }
+        return;
+    }
+    constexpr int V_MAX = 16;
+    constexpr int PER = 16 / sizeof(T);  // elements of a 16-byte store
+    const int slice = (rows + v_group - 1) / v_group;
+    const T* x0 = qkv + (size_t)first * row_stride + v_first;
+    for (int i = place * slice + threadIdx.x; i < min(rows, (place + 1) * slice); i += blockDim.x) {
+        __attribute__((aligned(16))) T vals[V_MAX];
+        const float add = b ? b[i] : 0.f;
+#pragma unroll
+        for (int j = 0; j < V_MAX; ++j)
+            vals[j] = j < v_group ? from_float<T>(to_float(x0[(size_t)j * row_stride + i]) + add) : T(0);
+        T* dst = v_pages + ((size_t)page * rows + i) * page_size + (off - place);
+#pragma unroll
+        for (int j = 0; j < V_MAX; j += PER)
+            if (j < v_group) *reinterpret_cast<uint4*>(dst + j) = *reinterpret_cast<const uint4*>(vals + j);
+    }
+}
 
 template <typename T>
 __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_kernel(
@@ -29,82 +77,152 @@ __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_kernel(
     const float* __restrict__ k_gain, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
     const int* __restrict__ block_table, int table_width, T* __restrict__ k_pages, T* __restrict__ v_pages,
-    int n_heads, int n_kv, int head_dim, int value_dim, int rotary_dim, int page_size) {
-    __shared__ float normed[QKP_WAVES][QKP_MAX_HEAD_DIM];
+    int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim, int rotary_dim, int page_size, int v_group) {
     const int n = blockIdx.x, wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE;
     const int pos = positions[n];
     const int half = rotary_dim / 2;
-    T* row = qkv + (size_t)n * row_stride;
-    const float* cs = cos_table ? cos_table + (size_t)pos * half : nullptr;
-    const float* sn = sin_table ? sin_table + (size_t)pos * half : nullptr;
     int page = -1, off = 0;
     if (n_kv > 0) {
         page = block_table[(size_t)seq_of_token[n] * table_width + pos / page_size];
         off = pos % page_size;
     }
     const int k_first = n_heads * head_dim, v_first = k_first + n_kv * head_dim;
-
-    const int total = n_heads + 2 * n_kv;
-    for (int first = 0; first < total; first += QKP_WAVES) {   // every wave takes every turn: the barriers are shared
-        const int item = first + wave;
-        const bool qk = item < n_heads + n_kv;
-        if (item < total && !qk && page >= 0) {   // a value head: bias, then into the page
-            const int h = item - n_heads - n_kv;
-            for (int d = lane; d < value_dim; d += SIA_WAVE) {
-                const int col = v_first + h * value_dim + d;
-                float v = to_float(row[col]);
-                if (bias) v += bias[col];
-                v_pages[(((size_t)page * n_kv + h) * value_dim + d) * page_size + off] = from_float<T>(v);
-            }
-        }
-        const bool is_q = item < n_heads;
-        const int h = is_q ? item : item - n_heads;
-        const int col0 = is_q ? h * head_dim : k_first + h * head_dim;
-        const float* gain = is_q ? q_gain : k_gain;
-        float x[QKP_MAX_HEAD_DIM / SIA_WAVE];
-        if (qk) {
-            float ss = 0.f;
-#pragma unroll
-            for (int j = 0; j < QKP_MAX_HEAD_DIM / SIA_WAVE; ++j) {
-                const int d = lane + j * SIA_WAVE;
-                x[j] = 0.f;
-                if (d < head_dim) {
-                    x[j] = to_float(row[col0 + d]);
-                    if (bias) x[j] += bias[col0 + d];
-                }
-                ss += x[j] * x[j];
-            }
-            if (gain) {
-                const float inv = rsqrtf(wave_sum(ss) / (float)head_dim + eps);
-#pragma unroll
-                for (int j = 0; j < QKP_MAX_HEAD_DIM / SIA_WAVE; ++j) {
-                    const int d = lane + j * SIA_WAVE;
-                    if (d < head_dim) x[j] = x[j] * inv * gain[d];
-                }
-            }
-            // the rotation's partner of an element lies in another lane: through the wave's row of LDS
-#pragma unroll
-            for (int j = 0; j < QKP_MAX_HEAD_DIM / SIA_WAVE; ++j) {
-                const int d = lane + j * SIA_WAVE;
-                if (d < head_dim) normed[wave][d] = x[j];
-            }
-        }
-        __syncthreads();
-        if (qk) {
-            T* dst = is_q ? row + col0
-                          : (page >= 0 ? k_pages + (((size_t)page * n_kv + h) * page_size + off) * head_dim : nullptr);
-#pragma unroll
-            for (int j = 0; j < QKP_MAX_HEAD_DIM / SIA_WAVE; ++j) {
-                const int d = lane + j * SIA_WAVE;
-                if (d >= head_dim) continue;
-                float v = x[j];
-                if (d < half) v = x[j] * cs[d] - normed[wave][d + half] * sn[d];
-                else if (d < rotary_dim) v = x[j] * cs[d - half] + normed[wave][d - half] * sn[d - half];
-                if (dst) dst[d] = from_float<T>(v);
-            }
-        }
-        __syncthreads();   // the rows of LDS are free for the next turn
+    const int qk_groups = (n_heads + n_kv + QKP_WAVES - 1) / QKP_WAVES;
+    if ((int)blockIdx.y >= qk_groups) {  // the token's values
+        if (page >= 0)
+            write_values<T>(qkv, row_stride, bias, positions, seq_of_token, v_pages, n, n_tokens, page, off, pos, v_first,
+                            n_kv * value_dim, page_size, v_group);
+        return;
     }
+    const int item = blockIdx.y * QKP_WAVES + wave;
+    if (item >= n_heads + n_kv) return;  // wave-uniform
+    T* row = qkv + (size_t)n * row_stride;
+    const bool is_q = item < n_heads;
+    const int h = is_q ? item : item - n_heads;
+    const int col0 = is_q ? h * head_dim : k_first + h * head_dim;
+    const float* gain = is_q ? q_gain : k_gain;
+    float x[QKP_PER_LANE];
+    float ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < QKP_PER_LANE; ++j) {
+        const int d = lane + j * SIA_WAVE;
+        x[j] = 0.f;
+        if (d < head_dim) {
+            x[j] = to_float(row[col0 + d]);
+            if (bias) x[j] += bias[col0 + d];
+        }
+        ss += x[j] * x[j];
+    }
+    if (gain) {
+        const float inv = rsqrtf(wave_sum(ss) / (float)head_dim + eps);
+#pragma unroll
+        for (int j = 0; j < QKP_PER_LANE; ++j) {
+            const int d = lane + j * SIA_WAVE;
+            if (d < head_dim) x[j] = x[j] * inv * gain[d];
+        }
+    }
+    T* dst = is_q ? row + col0
+                  : (page >= 0 ? k_pages + (((size_t)page * n_kv + h) * page_size + off) * head_dim : nullptr);
+#pragma unroll
+    for (int j = 0; j < QKP_PER_LANE; ++j) {
+        if (j * SIA_WAVE >= head_dim) break;  // wave-uniform: the exchanges below are taken by all lanes or by none
+        const int d = lane + j * SIA_WAVE;
+        // element d turns with element d + half (d < half) or d - half (half <= d < rotary_dim)
+        const int mate = d < half ? d + half : (d < rotary_dim ? d - half : d);
+        float other = 0.f;
+#pragma unroll
+        for (int jj = 0; jj < QKP_PER_LANE; ++jj) {
+            if (jj * SIA_WAVE >= head_dim) break;
+            const float got = __shfl(x[jj], mate % SIA_WAVE, SIA_WAVE);
+            if (mate / SIA_WAVE == jj) other = got;
+        }
+        if (d >= head_dim) continue;
+        float v = x[j];
+        if (d < half) v = x[j] * cos_table[(size_t)pos * half + d] - other * sin_table[(size_t)pos * half + d];
+        else if (d < rotary_dim) v = x[j] * cos_table[(size_t)pos * half + d - half] + other * sin_table[(size_t)pos * half + d - half];
+        if (dst) dst[d] = from_float<T>(v);
+    }
+}
+
+// The same for head sizes of 16, 32, 64, 128 or 256 with rotary_dim a multiple of 16: a lane takes 8 consecutive
+// elements with 16- and 32-byte accesses, a head is head_dim / 8 neighbouring lanes, a wave 64 / (head_dim / 8)
+// heads; sums and the rotation's partners cross lanes inside a head's group only.  All of a lane's loads are
+// independent of one another and issued before the first is used.
+template <typename T>
+__global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_vec_kernel(
+    T* __restrict__ qkv, int row_stride, const float* __restrict__ bias, const float* __restrict__ q_gain,
+    const float* __restrict__ k_gain, float eps, const float* __restrict__ cos_table,
+    const float* __restrict__ sin_table, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+    const int* __restrict__ block_table, int table_width, T* __restrict__ k_pages, T* __restrict__ v_pages,
+    int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim, int rotary_dim, int page_size, int v_group) {
+    const int n = blockIdx.x, wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE;
+    const int pos = positions[n];
+    const int half = rotary_dim / 2;
+    const int group = head_dim / 8, heads_a_wave = SIA_WAVE / group;   // lanes of a head; a power of two up to 32
+    const int k_first = n_heads * head_dim, v_first = k_first + n_kv * head_dim;
+    const int qk_groups = (n_heads + n_kv + QKP_WAVES * heads_a_wave - 1) / (QKP_WAVES * heads_a_wave);
+    if ((int)blockIdx.y >= qk_groups) {  // the token's values
+        const int page = block_table[(size_t)seq_of_token[n] * table_width + pos / page_size];
+        if (page >= 0)
+            write_values<T>(qkv, row_stride, bias, positions, seq_of_token, v_pages, n, n_tokens, page, pos % page_size,
+                            pos, v_first, n_kv * value_dim, page_size, v_group);
+        return;
+    }
+    const int item = (blockIdx.y * QKP_WAVES + wave) * heads_a_wave + lane / group;
+    const bool live = item < n_heads + n_kv;
+    const int it = live ? item : 0;      // lanes without a head go along (the exchanges are taken by all) and store nothing
+    const bool is_q = it < n_heads;
+    const int h = is_q ? it : it - n_heads;
+    const int d0 = (lane % group) * 8;
+    const int col = (is_q ? h * head_dim : k_first + h * head_dim) + d0;
+    T* row = qkv + (size_t)n * row_stride;
+    const bool turns = d0 < rotary_dim, low = d0 < half;
+    const int t0 = low ? d0 : d0 - half;   // where this piece's angles lie in the tables' row
+    Vec8<T> vx;
+    Vec8<float> vb, vg, vc, vs;
+    vx.load(row + col);
+    if (bias) vb.load(bias + col);
+    const float* gain = is_q ? q_gain : k_gain;
+    if (gain) vg.load(gain + d0);
+    if (turns) {
+        vc.load(cos_table + (size_t)pos * half + t0);
+        vs.load(sin_table + (size_t)pos * half + t0);
+    }
+    int page = -1;
+    if (!is_q) page = block_table[(size_t)seq_of_token[n] * table_width + pos / page_size];
+    float x[8], b[8], g[8], c[8], sn[8];
+    vx.get(x);
+    if (bias) {
+        vb.get(b);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] += b[i];
+    }
+    if (gain) {
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ss += x[i] * x[i];
+        for (int o = group / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, SIA_WAVE);   // fixed order inside the head's lanes
+        const float inv = rsqrtf(ss / (float)head_dim + eps);
+        vg.get(g);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] = x[i] * inv * g[i];
+    }
+    if (rotary_dim > 0) {   // wave-uniform: every lane takes the exchange
+        const int mate = turns ? (low ? lane + half / 8 : lane - half / 8) : lane;
+        float other[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) other[i] = __shfl(x[i], mate, SIA_WAVE);
+        if (turns) {
+            vc.get(c);
+            vs.get(sn);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[i] = low ? x[i] * c[i] - other[i] * sn[i] : x[i] * c[i] + other[i] * sn[i];
+        }
+    }
+    if (!live) return;
+    vx.set(x);
+    if (is_q) vx.store(row + col);
+    else if (page >= 0) vx.store(k_pages + (((size_t)page * n_kv + h) * page_size + pos % page_size) * head_dim + d0);
 }
 
 SIA_EXPORT int sia_qk_prepare_max_head_dim() { return QKP_MAX_HEAD_DIM; }
@@ -121,11 +239,26 @@ SIA_EXPORT int sia_qk_prepare(void* qkv, int row_stride, const float* bias, cons
     if ((q_gain == nullptr) != (k_gain == nullptr)) return SIA_BAD_ARGUMENT;
     if (n_kv > 0 && (!k_pages || !v_pages || !block_table || page_size <= 0)) return SIA_BAD_ARGUMENT;
     if (row_stride < n_heads * head_dim + n_kv * (head_dim + value_dim)) return SIA_BAD_ARGUMENT;
-    dim3 grid(n_tokens), block(QKP_WAVES * SIA_WAVE);
-#define LAUNCH(T)                                                                                                  \
-    hipLaunchKernelGGL(qk_prepare_kernel<T>, grid, block, 0, stream, (T*)qkv, row_stride, bias, q_gain, k_gain, eps, \
-                       cos_table, sin_table, positions, seq_of_token, block_table, table_width, (T*)k_pages,       \
-                       (T*)v_pages, n_heads, n_kv, head_dim, value_dim, rotary_dim, page_size)
+    if (n_heads + n_kv > 65535 * QKP_WAVES) return SIA_BAD_ARGUMENT;
+    // tokens whose values one workgroup writes together (0: every token its own); needs runs aligned to 16 bytes
+    const int v_group = (n_kv > 0 && n_tokens > 1 && page_size % 16 == 0) ? 16 : (n_kv > 0 && n_tokens > 1 && page_size % 8 == 0) ? 8 : 0;
+    const bool vec = (head_dim == 16 || head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256) &&
+                     rotary_dim % 16 == 0 && row_stride % 8 == 0;
+    const int heads_a_group = QKP_WAVES * (vec ? SIA_WAVE / (head_dim / 8) : 1);
+    dim3 grid(n_tokens, (n_heads + n_kv + heads_a_group - 1) / heads_a_group + (n_kv > 0 ? 1 : 0)), block(QKP_WAVES * SIA_WAVE);
+#define LAUNCH(T)                                                                                                    \
+    do {                                                                                                             \
+        if (vec)                                                                                                     \
+            hipLaunchKernelGGL(qk_prepare_vec_kernel<T>, grid, block, 0, stream, (T*)qkv, row_stride, bias, q_gain,  \
+                               k_gain, eps, cos_table, sin_table, positions, seq_of_token, block_table, table_width, \
+                               (T*)k_pages, (T*)v_pages, n_tokens, n_heads, n_kv, head_dim, value_dim, rotary_dim,   \
+                               page_size, v_group);                                                                  \
+        else                                                                                                         \
+            hipLaunchKernelGGL(qk_prepare_kernel<T>, grid, block, 0, stream, (T*)qkv, row_stride, bias, q_gain,      \
+                               k_gain, eps, cos_table, sin_table, positions, seq_of_token, block_table, table_width, \
+                               (T*)k_pages, (T*)v_pages, n_tokens, n_heads, n_kv, head_dim, value_dim, rotary_dim,   \
+                               page_size, v_group);                                                                  \
+    } while (0)
     if (dtype == SIA_F32) LAUNCH(float);
     else if (dtype == SIA_BF16) LAUNCH(bf16_t);
     else return SIA_BAD_ARGUMENT;

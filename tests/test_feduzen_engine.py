@@ -303,3 +303,32 @@ def test_trace_replay_of_a_model_folder_on_the_cpu(folders):
     assert F.rel_err(out, torch.stack([ra[39], rb[0], rb[32]])) < 3e-5
     assert F.rel_err(out2, torch.stack([ra[69], rb[1]])) < 3e-5
     assert not rp.ids and rp.cache.free_pages() == 12
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["b", "c"])
+def test_bfloat16_generation_from_replayed_graphs_is_the_eager_one(folders, name):
+    """The serving path: bfloat16, decode steps replayed from graphs, the host running ahead.  The tokens are those
+    of eager steps, and each is the plain implementation's best token or ties with it within bfloat16's reach."""
+    from simple_inference_amd import Engine, EngineConfig, SamplingParams
+    vocab = F.CONFIGS[name]["vocab"]
+    prompts = [random_tokens(vocab, n, seed=400 + n) for n in (45, 70, 9)]
+    runs = {}
+    for graphs in (True, False):
+        eng = Engine.from_folder(folders[name], EngineConfig(
+            device="cuda:0", dtype="bfloat16", max_seq_len=256, block_size=16, max_running=4, chunk_tokens=64,
+            eos_id=-1, use_graphs=graphs, run_ahead=graphs))
+        reqs = [eng.add_request(p, params=SamplingParams(temperature=0.0, max_new_tokens=40)) for p in prompts]
+        eng.run()
+        runs[graphs] = [list(r.generated) for r in reqs]
+        if graphs:
+            assert eng.graphs is not None and eng.stats["graph_fallbacks"] == 0
+    assert runs[True] == runs[False]
+    cfg, w = F.read_model(folders[name])
+    for prompt, generated in zip(prompts, runs[True]):
+        toks = list(prompt)
+        for got in generated:
+            logits = F.plain.forward(cfg, w, toks)[-1]
+            want = int(torch.argmax(logits))
+            assert got == want or float(logits[want] - logits[got]) < 4e-2 * float(logits.abs().max())
+            toks.append(got)
