@@ -15,6 +15,16 @@ _LLAMA3_SCALING_32 = {
     "high_freq_factor": 4.0, "original_max_position_embeddings": 8192,
 }
 
+def _feduzen_layer(ff, weights_of=None):
+    layer = {"type": "attention", "mlp": {"kind": "dense", "ff": ff} if ff else None,
+             "mixer": {"heads": 8, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.11, "mask": {"size": 256},
+                       "rot": {"dims": 32, "base": 100000.0,
+                               "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 1024}}}}
+    if weights_of is not None:
+        layer["weights_of"] = weights_of
+    return layer
+
+
 PRESETS = {
     "llama-3.2-3b": {
         "architectures": ["LlamaForCausalLM"], "model_type": "llama",
@@ -40,6 +50,12 @@ PRESETS = {
         "rope_scaling": dict(_LLAMA3_SCALING_32, factor=8.0),
         "max_position_embeddings": 131072, "bos_token_id": 128000, "eos_token_id": 128001,
         "tie_word_embeddings": False, "torch_dtype": "bfloat16", "hidden_act": "silu",
+    },
+    # a small model of the Feduzen design: five runs of three layers' weights, one layer without a feed-forward
+    "feduzen-small": {
+        "architecture": "Feduzen", "vocab": 4096, "width": 512, "embedding": {"scale": 2.0}, "norm": {"eps": 1e-6},
+        "layers": [_feduzen_layer(1536), _feduzen_layer(None), _feduzen_layer(None, weights_of=1),
+                   _feduzen_layer(1536), _feduzen_layer(1536, weights_of=0)],
     },
     "tiny-a": {
         "architectures": ["LlamaForCausalLM"], "model_type": "llama",
