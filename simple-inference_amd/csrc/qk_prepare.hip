@@ -13,8 +13,12 @@
 //
 // q is written back in place, k goes to the token's place in its page, v (with its bias) too.
 //
-// Page layout:  keys   [page][kv_head][offset][head_dim]
-//               values [page][kv_head][value_dim][offset]      (positions innermost)
+// Page layout:  keys   [page][kv_head][offset][k_row]
+//               values [page][kv_head][v_rows][offset]      (positions innermost)
+// k_row and v_rows are head_dim and value_dim, or larger: pages may be wider than the heads (a mixer whose keys and
+// values differ in width can keep both at one width, for kernels that want them alike); what lies beyond a head's
+// own elements is never written and stays as the pages were made (zero).  q goes back in place, or to a matrix of
+// its own with heads q_head_stride apart (the elements between heads are the caller's: zero).
 //
 // A wave takes one q or k head of one token: a lane holds the elements lane, lane + 64, ... of the head, the sum
 // of squares is a butterfly over the wave, and the rotation's partner of an element comes from the lane that holds
@@ -33,7 +37,10 @@ template <typename T>
 __device__ __forceinline__ void write_values(const T* __restrict__ qkv, int row_stride, const float* __restrict__ bias,
                                              const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                                              T* __restrict__ v_pages, int n, int n_tokens, int page, int off, int pos,
-                                             int v_first, int rows, int page_size, int v_group) {
+                                             int v_first, int rows, int value_dim, int v_rows, int page_size,
+                                             int v_group) {
+    const size_t page_rows = (size_t)(rows / value_dim) * v_rows;   // value rows of a page, over its kv heads
+    auto page_row = [&](int i) { return (size_t)(i / value_dim) * v_rows + i % value_dim; };
     const T* x = qkv + (size_t)n * row_stride + v_first;
     const float* b = bias ? bias + v_first : nullptr;
     bool whole = false;
@@ -50,7 +57,7 @@ __device__ __forceinline__ void write_values(const T* __restrict__ qkv, int row_
         for (int i = threadIdx.x; i < rows; i += blockDim.x) {
             float v = to_float(x[i]);
             if (b) v += b[i];
-            v_pages[((size_t)page * rows + i) * page_size + off] = from_float<T>(v);
+            v_pages[((size_t)page * page_rows + page_row(i)) * page_size + off] = from_float<T>(v);
         }
         return;
     }
@@ -64,7 +71,7 @@ __device__ __forceinline__ void write_values(const T* __restrict__ qkv, int row_
 #pragma unroll
         for (int j = 0; j < V_MAX; ++j)
             vals[j] = j < v_group ? from_float<T>(to_float(x0[(size_t)j * row_stride + i]) + add) : T(0);
-        T* dst = v_pages + ((size_t)page * rows + i) * page_size + (off - place);
+        T* dst = v_pages + ((size_t)page * page_rows + page_row(i)) * page_size + (off - place);
 #pragma unroll
         for (int j = 0; j < V_MAX; j += PER)
             if (j < v_group) *reinterpret_cast<uint4*>(dst + j) = *reinterpret_cast<const uint4*>(vals + j);
@@ -73,11 +80,12 @@ __device__ __forceinline__ void write_values(const T* __restrict__ qkv, int row_
 
 template <typename T>
 __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_kernel(
-    T* __restrict__ qkv, int row_stride, const float* __restrict__ bias, const float* __restrict__ q_gain,
+    T* qkv, int row_stride, const float* __restrict__ bias, const float* __restrict__ q_gain,
     const float* __restrict__ k_gain, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
     const int* __restrict__ block_table, int table_width, T* __restrict__ k_pages, T* __restrict__ v_pages,
-    int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim, int rotary_dim, int page_size, int v_group) {
+    int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim, int rotary_dim, int page_size, int v_group,
+    int k_row, int v_rows, T* q_out, int q_row_stride, int q_head_stride) {   // q_out may be qkv
     const int n = blockIdx.x, wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE;
     const int pos = positions[n];
     const int half = rotary_dim / 2;
@@ -91,7 +99,7 @@ __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_kernel(
     if ((int)blockIdx.y >= qk_groups) {  // the token's values
         if (page >= 0)
             write_values<T>(qkv, row_stride, bias, positions, seq_of_token, v_pages, n, n_tokens, page, off, pos, v_first,
-                            n_kv * value_dim, page_size, v_group);
+                            n_kv * value_dim, value_dim, v_rows, page_size, v_group);
         return;
     }
     const int item = blockIdx.y * QKP_WAVES + wave;
@@ -121,8 +129,8 @@ __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_kernel(
             if (d < head_dim) x[j] = x[j] * inv * gain[d];
         }
     }
-    T* dst = is_q ? row + col0
-                  : (page >= 0 ? k_pages + (((size_t)page * n_kv + h) * page_size + off) * head_dim : nullptr);
+    T* dst = is_q ? q_out + (size_t)n * q_row_stride + h * q_head_stride
+                  : (page >= 0 ? k_pages + (((size_t)page * n_kv + h) * page_size + off) * k_row : nullptr);
 #pragma unroll
     for (int j = 0; j < QKP_PER_LANE; ++j) {
         if (j * SIA_WAVE >= head_dim) break;  // wave-uniform: the exchanges below are taken by all lanes or by none
@@ -150,11 +158,12 @@ __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_kernel(
 // independent of one another and issued before the first is used.
 template <typename T>
 __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_vec_kernel(
-    T* __restrict__ qkv, int row_stride, const float* __restrict__ bias, const float* __restrict__ q_gain,
+    T* qkv, int row_stride, const float* __restrict__ bias, const float* __restrict__ q_gain,
     const float* __restrict__ k_gain, float eps, const float* __restrict__ cos_table,
     const float* __restrict__ sin_table, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
     const int* __restrict__ block_table, int table_width, T* __restrict__ k_pages, T* __restrict__ v_pages,
-    int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim, int rotary_dim, int page_size, int v_group) {
+    int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim, int rotary_dim, int page_size, int v_group,
+    int k_row, int v_rows, T* q_out, int q_row_stride, int q_head_stride) {   // q_out may be qkv
     const int n = blockIdx.x, wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE;
     const int pos = positions[n];
     const int half = rotary_dim / 2;
@@ -165,7 +174,7 @@ __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_vec_kernel(
         const int page = block_table[(size_t)seq_of_token[n] * table_width + pos / page_size];
         if (page >= 0)
             write_values<T>(qkv, row_stride, bias, positions, seq_of_token, v_pages, n, n_tokens, page, pos % page_size,
-                            pos, v_first, n_kv * value_dim, page_size, v_group);
+                            pos, v_first, n_kv * value_dim, value_dim, v_rows, page_size, v_group);
         return;
     }
     const int item = (blockIdx.y * QKP_WAVES + wave) * heads_a_wave + lane / group;
@@ -221,8 +230,8 @@ __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_vec_kernel(
     }
     if (!live) return;
     vx.set(x);
-    if (is_q) vx.store(row + col);
-    else if (page >= 0) vx.store(k_pages + (((size_t)page * n_kv + h) * page_size + pos % page_size) * head_dim + d0);
+    if (is_q) vx.store(q_out + (size_t)n * q_row_stride + h * q_head_stride + d0);
+    else if (page >= 0) vx.store(k_pages + (((size_t)page * n_kv + h) * page_size + pos % page_size) * k_row + d0);
 }
 
 SIA_EXPORT int sia_qk_prepare_max_head_dim() { return QKP_MAX_HEAD_DIM; }
@@ -231,7 +240,8 @@ SIA_EXPORT int sia_qk_prepare(void* qkv, int row_stride, const float* bias, cons
                               float eps, const float* cos_table, const float* sin_table, const int* positions,
                               const int* seq_of_token, const int* block_table, int table_width, void* k_pages,
                               void* v_pages, int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim,
-                              int rotary_dim, int page_size, int dtype, hipStream_t stream) {
+                              int rotary_dim, int page_size, int k_row, int v_rows, void* q_out, int q_row_stride,
+                              int q_head_stride, int dtype, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (head_dim <= 0 || head_dim > QKP_MAX_HEAD_DIM || value_dim <= 0 || n_heads < 0 || n_kv < 0) return SIA_BAD_ARGUMENT;
     if (rotary_dim < 0 || rotary_dim > head_dim || (rotary_dim & 1)) return SIA_BAD_ARGUMENT;
@@ -239,11 +249,19 @@ SIA_EXPORT int sia_qk_prepare(void* qkv, int row_stride, const float* bias, cons
     if ((q_gain == nullptr) != (k_gain == nullptr)) return SIA_BAD_ARGUMENT;
     if (n_kv > 0 && (!k_pages || !v_pages || !block_table || page_size <= 0)) return SIA_BAD_ARGUMENT;
     if (row_stride < n_heads * head_dim + n_kv * (head_dim + value_dim)) return SIA_BAD_ARGUMENT;
+    if (n_kv > 0 && (k_row < head_dim || v_rows < value_dim)) return SIA_BAD_ARGUMENT;
+    if (!q_out) {  // q goes back where it came from
+        q_out = qkv;
+        q_row_stride = row_stride;
+        q_head_stride = head_dim;
+    }
+    if (q_head_stride < head_dim || q_row_stride < n_heads * q_head_stride) return SIA_BAD_ARGUMENT;
     if (n_heads + n_kv > 65535 * QKP_WAVES) return SIA_BAD_ARGUMENT;
     // tokens whose values one workgroup writes together (0: every token its own); needs runs aligned to 16 bytes
     const int v_group = (n_kv > 0 && n_tokens > 1 && page_size % 16 == 0) ? 16 : (n_kv > 0 && n_tokens > 1 && page_size % 8 == 0) ? 8 : 0;
     const bool vec = (head_dim == 16 || head_dim == 32 || head_dim == 64 || head_dim == 128 || head_dim == 256) &&
-                     rotary_dim % 16 == 0 && row_stride % 8 == 0;
+                     rotary_dim % 16 == 0 && row_stride % 8 == 0 && q_row_stride % 8 == 0 && q_head_stride % 8 == 0 &&
+                     k_row % 8 == 0;
     const int heads_a_group = QKP_WAVES * (vec ? SIA_WAVE / (head_dim / 8) : 1);
     dim3 grid(n_tokens, (n_heads + n_kv + heads_a_group - 1) / heads_a_group + (n_kv > 0 ? 1 : 0)), block(QKP_WAVES * SIA_WAVE);
 #define LAUNCH(T)                                                                                                    \
@@ -252,12 +270,12 @@ SIA_EXPORT int sia_qk_prepare(void* qkv, int row_stride, const float* bias, cons
             hipLaunchKernelGGL(qk_prepare_vec_kernel<T>, grid, block, 0, stream, (T*)qkv, row_stride, bias, q_gain,  \
                                k_gain, eps, cos_table, sin_table, positions, seq_of_token, block_table, table_width, \
                                (T*)k_pages, (T*)v_pages, n_tokens, n_heads, n_kv, head_dim, value_dim, rotary_dim,   \
-                               page_size, v_group);                                                                  \
+                               page_size, v_group, k_row, v_rows, (T*)q_out, q_row_stride, q_head_stride);           \
         else                                                                                                         \
             hipLaunchKernelGGL(qk_prepare_kernel<T>, grid, block, 0, stream, (T*)qkv, row_stride, bias, q_gain,      \
                                k_gain, eps, cos_table, sin_table, positions, seq_of_token, block_table, table_width, \
                                (T*)k_pages, (T*)v_pages, n_tokens, n_heads, n_kv, head_dim, value_dim, rotary_dim,   \
-                               page_size, v_group);                                                                  \
+                               page_size, v_group, k_row, v_rows, (T*)q_out, q_row_stride, q_head_stride);           \
     } while (0)
     if (dtype == SIA_F32) LAUNCH(float);
     else if (dtype == SIA_BF16) LAUNCH(bf16_t);

@@ -31,7 +31,8 @@ _SIGNATURES = {
     "sia_norm_add": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "sia_activation": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_ptr],
     "sia_qk_prepare": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
-                       _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+                       _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr,
+                       _c_int, _c_int, _c_int, _c_ptr],
     "sia_qk_prepare_max_head_dim": [],
     "sia_gemm_skinny_act": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_add_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
@@ -559,20 +560,35 @@ class HipKernels:
             "rope_kv_write")
 
     def qkv_to_cache(self, x, w_qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache,
-                     value_dim=None, bias=None, qk_norm=None):
+                     value_dim=None, bias=None, qk_norm=None, page_dim=None):
         """The q/k/v product, the rotation of q and k and the write of k and v into the pages.  Returns the
         ``[tokens, (n_heads + 2 n_kv_written) head_dim]`` matrix whose q columns hold the rotated queries; its
         k and v columns are not to be read (for few rows one kernel does all three and never writes them).
 
         ``value_dim``: width of a v head if not ``head_dim``; ``bias``: float ``[row width]``, added to the product;
         ``qk_norm``: ``(q_gain, k_gain, eps)``, an RMS norm over every q and k head before the rotation.  With any
-        of these the product is followed by one kernel that does all of bias, norm, rotation and cache write."""
+        of these the product is followed by one kernel that does all of bias, norm, rotation and cache write.
+
+        ``page_dim`` (see ``attention_page_dim``): the pages' keys and values are both that wide; the result is then
+        ``[tokens, n_heads * page_dim]``, the queries with zeros behind every head, and attention is called with
+        ``page_dim`` for the head size."""
         M, K = x.shape
-        if value_dim is not None or bias is not None or qk_norm is not None:
+        if value_dim is not None or bias is not None or qk_norm is not None or page_dim is not None:
             qkv = self.linear(x, w_qkv)
+            q_out = None
+            if page_dim is not None:
+                # one matrix a step and geometry, shared by the step's layers: its zeros between the heads are written
+                # once, the kernel only ever writes the heads' own elements
+                kept = getattr(ctx, "padded_queries", None)
+                if kept is None:
+                    kept = ctx.padded_queries = {}
+                key = (n_heads, page_dim, qkv.dtype)
+                q_out = kept.get(key)
+                if q_out is None:
+                    q_out = kept[key] = torch.zeros((M, n_heads * page_dim), dtype=qkv.dtype, device=qkv.device)
             self.qk_prepare(qkv, n_heads, n_kv_written, head_dim, value_dim or head_dim, rotary_dim, cos, sin, bias,
-                            qk_norm, ctx, cache)
-            return qkv
+                            qk_norm, ctx, cache, page_dim, q_out)
+            return qkv if q_out is None else q_out
         if (self.use_skinny_gemm and self.fuse_rope and n_kv_written and x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16
                 and M <= self._skinny_rows and rotary_dim == head_dim and head_dim % 2 == 0 and K % 64 == 0):
             x, partials, n_partials, norm_eps = self._scaled(x)
@@ -602,8 +618,21 @@ class HipKernels:
         self.rope_kv_write(qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache)
         return qkv
 
+    def attention_page_dim(self, head_dim: int, value_dim: int, dtype):
+        """The one width at which a mixer should keep both its keys and its values in the pages so that the
+        matrix-core attention kernel, which is compiled for one head size, can run on them; None where the pages can
+        be as wide as the heads are (the widths are alike and a multiple of 16, or no such kernel would run
+        anyway).  The elements beyond a head's own are zero: a zero in a key adds nothing to a score, a zero row of
+        values gives a zero that the output projection, widened by as many zero columns, ignores."""
+        if dtype != torch.bfloat16:
+            return None
+        wide = -(-max(head_dim, value_dim) // 16) * 16
+        if (wide == head_dim and wide == value_dim) or wide > 256:
+            return None
+        return wide
+
     def qk_prepare(self, qkv, n_heads, n_kv_written, head_dim, value_dim, rotary_dim, cos, sin, bias, qk_norm, ctx,
-                   cache):
+                   cache, page_dim=None, q_out=None):
         """Bias, per-head RMS norm of q and k, rotation, and the write of k and v into the pages, on the projected
         rows ``[q heads | k heads | v heads]`` (q and k heads ``head_dim`` wide, v heads ``value_dim``); q is left in
         place."""
@@ -634,14 +663,21 @@ class HipKernels:
             self._want(k_gain, "k norm gain", torch.float32, (head_dim,))
         table = k_pages = v_pages = None
         page_size = 0
+        k_row, v_rows = head_dim, value_dim
+        if page_dim is not None:
+            if page_dim < max(head_dim, value_dim) or q_out is None:
+                raise KernelError(f"pages of width {page_dim} do not hold heads of {head_dim} and values of {value_dim}")
+            self._want(q_out, "padded queries", qkv.dtype, (n, n_heads * page_dim))
+            k_row = v_rows = page_dim
         if n_kv_written:
             k_pages, v_pages, table, page_size = cache.k_pages, cache.v_pages, cache.block_table, cache.page_size
-            self._check_pages(k_pages, v_pages, table, page_size, n_kv_written, head_dim, qkv.dtype, ctx, value_dim)
+            self._check_pages(k_pages, v_pages, table, page_size, n_kv_written, k_row, qkv.dtype, ctx, v_rows)
         self._check(self.core.sia_qk_prepare(
             _ptr(qkv), width, _ptr(bias), _ptr(q_gain), _ptr(k_gain), float(eps),
             _ptr(cos) if rotary_dim else None, _ptr(sin) if rotary_dim else None, _ptr(ctx.positions),
             _ptr(ctx.seq_of_token), _ptr(table), table.shape[1] if table is not None else 0, _ptr(k_pages),
-            _ptr(v_pages), n, n_heads, n_kv_written, head_dim, value_dim, rotary_dim, page_size, _DT[qkv.dtype],
+            _ptr(v_pages), n, n_heads, n_kv_written, head_dim, value_dim, rotary_dim, page_size, k_row, v_rows,
+            _ptr(q_out), n_heads * page_dim if page_dim else 0, page_dim or 0, _DT[qkv.dtype],
             self._stream()), "qk_prepare")
 
     def _check_pages(self, k_pages, v_pages, table, page_size, n_kv, head_dim, dtype, ctx, value_dim=None):

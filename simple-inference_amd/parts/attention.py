@@ -83,6 +83,9 @@ class Attention:
         check = getattr(env.kernels, "check_attention_geometry", None)
         if check is not None:     # sizes the kernels refuse are refused here, when the model is built
             check(self.num_heads, self.num_kv_heads, max(self.head_dim, self.value_dim))
+        # kernels that want keys and values of one width say at which width this mixer should keep its pages
+        page_dim = getattr(env.kernels, "attention_page_dim", None)
+        self.page_dim = page_dim(self.head_dim, self.value_dim, env.dtype) if page_dim is not None and self._options() else None
         self.env = env
         self.w_qkv = None
         self.w_o = None
@@ -117,6 +120,10 @@ class Attention:
         else:
             self.w_qkv = tensors["q"].contiguous()
         self.w_o = tensors["o"].contiguous()
+        if self.page_dim is not None:   # the attention's rows come with page_dim elements a head: zero columns for the rest
+            wide = self.w_o.new_zeros((self.hidden, self.num_heads, self.page_dim))
+            wide[:, :, :self.value_dim] = self.w_o.view(self.hidden, self.num_heads, self.value_dim)
+            self.w_o = wide.view(self.hidden, self.num_heads * self.page_dim)
         if self.bias:
             self.b_qkv = torch.cat([tensors["q_bias"], tensors["k_bias"], tensors["v_bias"]]).contiguous()
         if self.qk_norm_eps is not None:
@@ -144,6 +151,8 @@ class Attention:
                 or self.value_dim != self.head_dim)
 
     def cache_need(self):
+        if self.page_dim is not None:
+            return PagedKVNeed(self.num_kv_heads, self.page_dim, self.window, None, self.chunk)
         return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window,
                            self.value_dim if self.value_dim != self.head_dim else None, self.chunk)
 
@@ -156,7 +165,11 @@ class Attention:
         project, attend = {}, {}
         if self._options():   # only then: a kernels object that knows none of these forms serves the plain mixer
             if self.value_dim != self.head_dim:
-                project["value_dim"] = attend["value_dim"] = self.value_dim
+                project["value_dim"] = self.value_dim
+                if self.page_dim is None:
+                    attend["value_dim"] = self.value_dim
+            if self.page_dim is not None:
+                project["page_dim"] = self.page_dim
             if self.bias:
                 project["bias"] = self.b_qkv
             if self.qk_norm_eps is not None:
@@ -169,5 +182,6 @@ class Attention:
             h, self.w_qkv, self.num_heads, self.num_kv_heads if self.writes_kv else 0, self.head_dim,
             self.position.rotary_dim, cos, sin, ctx, cache, **project)
         out = k.paged_attention(
-            qkv, self.num_heads, self.num_kv_heads, self.head_dim, self.scale, self.window, ctx, cache, **attend)
+            qkv, self.num_heads, self.num_kv_heads, self.page_dim or self.head_dim, self.scale, self.window, ctx, cache,
+            **attend)
         return k.pending_linear(out, self.w_o)   # the norm after it may have it added into the residual

@@ -310,3 +310,41 @@ def test_the_sink_takes_weight_and_gives_nothing(backend):
     got = k.paged_attention(qkv.to(dev), heads, kv, dim, 0.2, None, ctx, cache, sinks=torch.zeros(heads).to(dev))
     first = got.view(-1, heads, dim).float().cpu()[0]       # the single token at position L - 1 sees L keys
     close(first[0], values[:, 0].mean(0) * L / (L + 1), backend)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("backend", ["hip-f32", "hip-bf16"])
+@pytest.mark.parametrize("heads,kv,dim,vdim,rot,wide", [(3, 3, 32, 16, 32, 32), (4, 2, 16, 48, 8, 48), (2, 2, 24, 24, 0, 32),
+                                                        (5, 1, 80, 40, 80, 80), (2, 1, 64, 128, 32, 128)])
+def test_pages_wider_than_the_heads_hold_the_same_numbers_and_zeros(backend, heads, kv, dim, vdim, rot, wide):
+    """Keys and values kept at one width (for the attention kernel that wants them alike): the heads' own elements
+    are what they are in pages as wide as the heads, everything beyond them is zero, and attention over such pages
+    gives the same result with zeros behind every head."""
+    k, dev, dtype = setup(backend)
+    page = 16
+    ctx, table, n_pages, runs = step_context(dev, [(40, 1), (0, 37), (21, 19)], page, k)
+    N, width = ctx.n_tokens, heads * dim + kv * (dim + vdim)
+    qkv0 = rnd(N, width, seed=80).to(dtype).to(dev)
+    bias, qg, kg = rnd(width, seed=81, std=0.5).to(dev), (1 + rnd(dim, seed=82, std=0.3)).to(dev), (1 + rnd(dim, seed=83, std=0.3)).to(dev)
+    cos, sin = rope_tables(rot, 500.0, None, 64, dev) if rot else (None, None)
+    eye = torch.eye(width).to(dtype).to(dev)
+    plain_cache = empty_cache(dev, dtype, n_pages, kv, page, dim, vdim, table)
+    wide_cache = empty_cache(dev, dtype, n_pages, kv, page, wide, wide, table)
+    q1 = k.qkv_to_cache(qkv0, eye, heads, kv, dim, rot, cos, sin, ctx, plain_cache, value_dim=vdim, bias=bias,
+                        qk_norm=(qg, kg, 1e-5))
+    q2 = k.qkv_to_cache(qkv0, eye, heads, kv, dim, rot, cos, sin, ctx, wide_cache, value_dim=vdim, bias=bias,
+                        qk_norm=(qg, kg, 1e-5), page_dim=wide)
+    assert tuple(q2.shape) == (N, heads * wide)
+    assert torch.equal(q2.view(N, heads, wide)[:, :, :dim], q1[:, :heads * dim].view(N, heads, dim))
+    assert float(q2.view(N, heads, wide)[:, :, dim:].abs().sum()) == 0
+    assert torch.equal(wide_cache.k_pages[..., :dim], plain_cache.k_pages) and float(wide_cache.k_pages[..., dim:].abs().sum()) == 0
+    assert torch.equal(wide_cache.v_pages[:, :, :vdim], plain_cache.v_pages) and float(wide_cache.v_pages[:, :, vdim:].abs().sum()) == 0
+    # fill the pasts of the runs that do not start at 0, alike in both
+    for cache in (plain_cache, wide_cache):
+        cache.k_pages[..., :dim] += 0.1
+        cache.v_pages[:, :, :vdim] += 0.2
+    sinks = rnd(heads, seed=84).to(dev)
+    o1 = k.paged_attention(q1, heads, kv, dim, 0.2, None, ctx, plain_cache, value_dim=vdim, chunk=30, sinks=sinks)
+    o2 = k.paged_attention(q2, heads, kv, wide, 0.2, None, ctx, wide_cache, chunk=30, sinks=sinks)
+    close(o2.view(N, heads, wide)[:, :, :vdim], o1.view(N, heads, vdim), backend)
+    assert float(o2.view(N, heads, wide)[:, :, vdim:].abs().sum()) == 0
