@@ -1,11 +1,11 @@
 """Typed configuration of the Feduzen design, read from its own config.json keys.
 
 A Feduzen config.json names the design in ``architecture`` and describes every layer in ``layers``: the kind of
-its mixer (``type``), the mixer's sizes and constants (``mixer``) and its feed-forward (``mlp``, or null).  A layer
-with ``weights_of: j`` has no tensors of its own and uses layer ``j``'s, with a cache of its own; what else its
-entry says must equal layer ``j``'s entry.  Every size and constant comes from here; nothing is derived from
-another model's habits (the score scale, the value width and the rotated width are all given, not implied by the
-head size).
+its mixer (``type``), the mixer's sizes and constants (``mixer``) and its feed-forward (``mlp``, or null).  An entry
+with ``weights_of: j`` stands for one more run of layer ``j``'s tensors (the checkpoint holds none under its index)
+that keeps separate keys and values; its description has to repeat layer ``j``'s, and is checked against it.
+Every size and constant comes from here; nothing is derived from another model's habits (the score scale, the
+value width and the rotated width are all given, not implied by the head size).
 """
 
 from __future__ import annotations

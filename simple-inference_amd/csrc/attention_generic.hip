@@ -9,11 +9,11 @@
 //
 //   s_j = (q . k_j) * scale                                   scale after the dot
 //   visible: j <= pos, and j > pos - window if window > 0, and j >= pos - pos % chunk if chunk > 0
-//            (blocks of chunk positions counted from position 0: a query sees its own block only)
+//            (absolute positions are cut into blocks [b * chunk, (b + 1) * chunk): causal inside the block)
 //   online softmax over chunks: m' = max(m, max_j s_j); p_j = exp(s_j - m');
 //   l = l * exp(m - m') + sum_j p_j;  acc = acc * exp(m - m') + sum_j p_j v_j;  o = acc / l
-//   with sinks: l += exp(sink_h - m) at the end, one learned number per query head that has no key and no
-//   value and is not scaled
+//   with sinks: l += exp(sink_h - m) at the end; sink_h is a learned logit of query head h that takes a share
+//   of the weight and carries no value (scale applies to the dot products only)
 // Values may have another width (value_dim) than keys and queries (head_dim).
 // (reference: kernels/attention_kernel.py:184-251, :516-586).  Everything is float.
 #include "common.h"

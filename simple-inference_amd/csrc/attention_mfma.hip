@@ -71,15 +71,15 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 constexpr float LOG2E = 1.4426950408889634f;
 
 // The oldest key a query at `pos` sees: all (window = chunk = 0), the last `window`, and/or those of its own block
-// of `chunk` positions (blocks counted from position 0).  It never falls as pos grows.
+// of `chunk` absolute positions [b * chunk, (b + 1) * chunk).  It never falls as pos grows.
 __device__ __forceinline__ int first_visible(int pos, int window, int chunk) {
     int lo = window > 0 ? max(0, pos - window + 1) : 0;
     if (chunk > 0) lo = max(lo, pos - pos % chunk);
     return lo;
 }
 
-// A sink's term of a softmax denominator: sinks[head] is one more score of that query head (natural units, not
-// scaled) that has no key and no value.  Exponentials are taken as 2^(x - ref) with ref in units of log2.
+// A sink's term of a softmax denominator: sinks[head] is a learned logit of that query head (natural units; the
+// score scale does not apply) that takes a share of the weight and carries no value.  Exponentials are taken as 2^(x - ref) with ref in units of log2.
 __device__ __forceinline__ float sink_term(const float* __restrict__ sinks, int head, float ref) {
     return sinks ? fast_exp2(sinks[head] * LOG2E - ref) : 0.f;
 }

@@ -7,8 +7,9 @@ a per-head RMS norm of q and k before a rotation of the first ``rot.dims`` dimen
 a mask of blocks of ``mask.size`` positions, and a per-head sink in the softmax; its feed-forward is dense with
 the square of relu.  The embedding is multiplied by ``embedding.scale``; the head has a matrix of its own.
 
-A layer with ``weights_of`` runs another layer's parts once more, with a cache of its own: in the plan it is a
-second entry of ``order`` for that layer, not a second copy of its tensors.
+A layer with ``weights_of`` is a further run of the parts of the layer it names, and its keys and values go to
+pages that only this run uses: in the plan it is a second entry of ``order`` for that layer, not a second copy of
+its tensors.
 
 Checkpoint names: ``embed``, ``final.norm``, ``head``; layer ``i``: ``l<i>.norm1``, ``l<i>.norm2``,
 ``l<i>.mix.{q,k,v}`` with ``.b`` for the biases, ``l<i>.mix.{q,k}.norm``, ``l<i>.mix.sink``, ``l<i>.mix.o``,

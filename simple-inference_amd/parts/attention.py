@@ -21,10 +21,12 @@ Further forms, each switched on by a parameter of its own and free to combine:
 * ``qk_norm`` (``{"eps": e}``): every q and k head is divided by its root mean square over the head
   (``x / sqrt(mean(x^2) + e)``) and multiplied by a gain of size ``D`` that all heads share (one for q, one for k),
   after the bias and before the rotation.
-* ``chunk``: position ``p`` sees key ``j <= p`` only if both lie in the same block of ``chunk`` positions, blocks
-  counted from position 0 of the sequence.
-* ``sink``: one learned number per query head joins the softmax's denominator as ``exp(sink_h)``; it has no key,
-  no value and is not scaled.
+* ``chunk``: the sequence's absolute positions are cut into blocks ``[b*chunk, (b+1)*chunk)``; a query attends
+  causally inside its block and to nothing before the block's first position (how a prompt was fed in portions
+  does not move the blocks).
+* ``sink``: a learned logit per query head that competes in the softmax but carries no value: the weights of
+  the real keys are ``exp(s_j) / (sum_i exp(s_i) + exp(sink_h))``, with ``sink_h`` taken as it is (``scale``
+  applies to the dot products only).
 """
 
 from __future__ import annotations

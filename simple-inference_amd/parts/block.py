@@ -5,8 +5,8 @@ Pre-norm (reference: ``model/block.py:135-147``):
 as the stream's pending delta and summed into the float32 residual by the norm
 that follows (the next layer's, or the model's last norm).
 
-Output-norm: ``x += norm1(mixer(x))``; ``x += norm2(feed_forward(x))``.  The sublayers read the residual itself
-(rounded to the compute dtype) and the norm sits on what a sublayer returns; the kernel that adds the normed
+Output-norm: ``x += norm1(mixer(x))``; ``x += norm2(feed_forward(x))``.  Mixer and feed-forward take the
+un-normed stream as input (rounded to the compute dtype), and each norm is applied to its sublayer's result; the kernel that adds the normed
 output into the float32 residual also leaves the rounded residual for the next sublayer.  A layer of this kind
 may have no feed-forward.
 """

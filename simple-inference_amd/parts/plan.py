@@ -118,8 +118,7 @@ class TensorSpec:
 @dataclass(frozen=True)
 class PagedKVNeed:
     """Keys and values in pages: all keys (``window`` and ``chunk`` None), the last ``window``, or those of the
-    current block of ``chunk`` positions (blocks counted from position 0: a query at ``p`` sees nothing below
-    ``p - p % chunk``).
+    current block of ``chunk`` absolute positions (a query at ``p`` sees nothing below ``p - p % chunk``).
 
     A page holds, per key/value head, ``page_size`` key rows of ``head_dim`` elements and as many value rows of
     ``value_head_dim`` elements (None: the same width).  The cache manager only stores them; what a row means is

@@ -5,8 +5,8 @@ checkpoint names and computes everything in float64 (or whatever dtype its tenso
 compare the engine with it.
 
 Notation.  ``x`` is the residual stream ``[T, width]`` of one sequence whose tokens stand at positions
-``0 .. T-1``.  A layer is ``x += N1(mixer(x))`` and, if it has a feed-forward, ``x += N2(ff(x))``: the norm sits on
-what a sublayer *returns*, and the sublayers read ``x`` as it is.
+``0 .. T-1``.  A layer is ``x += N1(mixer(x))`` and, if it has a feed-forward, ``x += N2(ff(x))``: each norm is
+applied to its sublayer's result, and mixer and feed-forward get the stream un-normed.
 """
 
 from __future__ import annotations
@@ -59,8 +59,8 @@ def rotate(x, positions, dims, base, scaling=None):
 
 
 def chunk_mask(n, size):
-    """``[n, n]`` bool: key ``j`` is seen from ``i`` iff ``j <= i`` and both lie in the same block of ``size``
-    positions counted from 0 (``size`` None: plain causal)."""
+    """``[n, n]`` bool: key ``j`` is seen from ``i`` iff ``j <= i`` and ``j // size == i // size`` (``size`` None:
+    plain causal)."""
     i = torch.arange(n)[:, None]
     j = torch.arange(n)[None, :]
     seen = j <= i
@@ -70,7 +70,7 @@ def chunk_mask(n, size):
 
 
 def softmax_with_sink(scores, sink):
-    """Softmax over the last axis whose denominator holds one more term ``exp(sink)``, which has no value."""
+    """Softmax over the last axis with ``exp(sink)`` added to the denominator and to nothing else."""
     m = torch.maximum(scores.max(-1, keepdim=True).values, sink)
     e = torch.exp(scores - m)
     return e / (e.sum(-1, keepdim=True) + torch.exp(sink - m))

@@ -305,7 +305,7 @@ def test_the_sink_takes_weight_and_gives_nothing(backend):
     for h in (2, 3):   # the values are near 1: the sink's share of the weight is what is missing
         share = 1 - a[:, h].mean(-1) / b[:, h].mean(-1)
         assert float(share.min()) > 0.001 and float(share.max()) < 0.999
-    # a sink is not scaled: with a sink of zero and scores of zero (no query) it is one more among n + 1
+    # the score scale does not touch a sink: with a sink of zero and scores of zero (no query) it is one among n + 1
     qkv.zero_()
     got = k.paged_attention(qkv.to(dev), heads, kv, dim, 0.2, None, ctx, cache, sinks=torch.zeros(heads).to(dev))
     first = got.view(-1, heads, dim).float().cpu()[0]       # the single token at position L - 1 sees L keys
