@@ -445,6 +445,19 @@ SIA_EXPORT int sia_gemm_skinny_residual_tiled(const void* X, const void* W_tiled
     return SIA_LAUNCH_CHECK();
 }
 
+// Y[M, N] = X W^T (bfloat16) from the tiled copy of W: the plain product for a weight that has such a copy, with the
+// sums of sia_gemm_skinny bit for bit.  Needs M <= 16, K % 64 == 0, sia_gemm_skinny_tile_height(N) > 0.
+SIA_EXPORT int sia_gemm_skinny_tiled(const void* X, const void* W_tiled, void* Y, int M, int N, int K,
+                                     hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (M > 16 || K % 64 || K <= 0 || !Y) return SIA_BAD_ARGUMENT;
+    const Cut cut = cheapest(N, 1, {4, 2, 1});
+    if (cut.unit_blocks != 1) return SIA_BAD_ARGUMENT;
+    hipLaunchKernelGGL((gemm_skinny_kernel<bf16_t, 1, 8, EPI_STORE, false, true>), dim3(cut.grid), dim3(8 * SIA_WAVE), 0,
+                       stream, (const bf16_t*)X, (const bf16_t*)W_tiled, (bf16_t*)Y, M, N, K, cut.bh, Epilogue{});
+    return SIA_LAUNCH_CHECK();
+}
+
 // Y[M, I] = silu(X Wg^T) * (X Wu^T) for W = [Wg; Wu] of 2 I rows.  Needs M <= 16, K % 64 == 0.
 // With `partials` (else null) X is a `scaled` matrix of sia_gemm_skinny_residual and the rows are divided by their
 // root mean square first.

@@ -60,6 +60,7 @@ _SIGNATURES = {
     "sia_gemm_skinny_residual": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "sia_gemm_skinny_residual_tiled": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr],
     "sia_gemm_skinny_tile_height": [_c_int],
+    "sia_gemm_skinny_tiled": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "sia_place_tokens": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr],
     "sia_scale_rows": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_ptr],
     "sia_stream_read": [_c_ptr, _c_ll, _c_ptr, _c_ptr],
@@ -352,6 +353,11 @@ class HipKernels:
             # up to 16 rows: this package's kernel, whose sums do not depend on the number of rows
             if self.use_skinny_gemm and M <= self._skinny_rows and K % 64 == 0:
                 y = torch.empty((M, N), dtype=torch.float32 if out_float32 else torch.bfloat16, device=x.device)
+                tiled = None if out_float32 else self._tiled_copy(w)
+                if tiled is not None:   # a weight that has a copy in the order of this kernel's loads: the same bits
+                    self._check(self.core.sia_gemm_skinny_tiled(_ptr(x), _ptr(tiled), _ptr(y), M, N, K, self._stream()),
+                                "gemm_skinny_tiled")
+                    return y
                 self._check(self.core.sia_gemm_skinny(_ptr(x), _ptr(w), _ptr(y), M, N, K, int(out_float32),
                                                       self._stream()), "gemm_skinny")
                 return y

@@ -33,6 +33,9 @@ class DenseFeedForward:
     def bind(self, tensors):
         self.w_up = tensors["up"].contiguous()
         self.w_down = tensors["down"].contiguous()
+        prepare = getattr(self.env.kernels, "prepare_pending_weight", None)
+        if prepare is not None:   # the kernels may keep a copy of their own of a weight for their few-row product
+            prepare(self.w_down)
 
     def forward(self, h, ctx):
         k = self.env.kernels

@@ -348,3 +348,16 @@ def test_pages_wider_than_the_heads_hold_the_same_numbers_and_zeros(backend, hea
     o2 = k.paged_attention(q2, heads, kv, wide, 0.2, None, ctx, wide_cache, chunk=30, sinks=sinks)
     close(o2.view(N, heads, wide)[:, :, :vdim], o1.view(N, heads, vdim), backend)
     assert float(o2.view(N, heads, wide)[:, :, vdim:].abs().sum()) == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("rows,n,k", [(1, 3072, 8192), (8, 3072, 3072), (16, 320, 384), (5, 200, 128)])
+def test_few_row_product_from_the_tiled_copy_of_a_weight_has_the_same_bits(rows, n, k):
+    kern, dev, _ = setup("hip-bf16")
+    x, w = rnd(rows, k, seed=90).bfloat16().to(dev), rnd(n, k, seed=91, std=0.05).bfloat16().to(dev)
+    plain_y = kern.linear(x, w)
+    made = kern.prepare_pending_weight(w)
+    assert made == (kern.core.sia_gemm_skinny_tile_height(n) > 0)
+    tiled_y = kern.linear(x, w)
+    assert torch.equal(plain_y, tiled_y)
+    close(tiled_y, x.double() @ w.double().T, "hip-bf16")
