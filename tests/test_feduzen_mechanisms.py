@@ -361,3 +361,96 @@ def test_few_row_product_from_the_tiled_copy_of_a_weight_has_the_same_bits(rows,
     tiled_y = kern.linear(x, w)
     assert torch.equal(plain_y, tiled_y)
     close(tiled_y, x.double() @ w.double().T, "hip-bf16")
+
+
+def fill_cache_by_pages(cache, table, keys, values, page, s):
+    """As ``fill_cache``, a page at a time (for long sequences)."""
+    L, kv, dim = keys.shape
+    n = -(-L // page)
+    k = torch.zeros(n * page, kv, dim, dtype=keys.dtype)
+    v = torch.zeros(n * page, kv, values.shape[2], dtype=values.dtype)
+    k[:L], v[:L] = keys, values
+    pages = table[s, :n].long()
+    cache.k_pages[pages] = k.view(n, page, kv, dim).permute(0, 2, 1, 3).to(cache.k_pages.dtype).to(cache.k_pages.device)
+    cache.v_pages[pages] = v.view(n, page, kv, -1).permute(0, 2, 3, 1).to(cache.v_pages.dtype).to(cache.v_pages.device)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n_seqs,mode", [(4, 2), (40, 0), (130, 1)])
+@pytest.mark.parametrize("chunk", [None, 2048])
+def test_sinks_and_blocks_where_decode_attention_splits_the_keys(n_seqs, mode, chunk):
+    """Long contexts in bfloat16: a sequence's keys are shared by several workgroups and their partial results are
+    merged (by the kernel that combines splits, by the one that combines every run, or inside one workgroup,
+    depending on how many sequences the step holds).  The sink joins the merged denominator exactly once."""
+    k, dev, dtype = setup("hip-bf16")
+    heads, kv, dim, page, scale = 8, 2, 64, 16, 0.11
+    lengths = [(2500, 1100, 3000, 600, 1025, 2049)[i % 6] for i in range(n_seqs)]
+    ctx, table, n_pages, runs = step_context(dev, [(L - 1, 1) for L in lengths], page, k)
+    lib = k._attn_lib(dim)
+    splits = lib.sia_attn_decode_max_splits(max(lengths), chunk or 0)
+    assert splits > 1 and lib.sia_attn_decode_mode(n_seqs, heads, kv, splits) == mode
+    cache = empty_cache(dev, dtype, n_pages, kv, page, dim, dim, table)
+    sinks = torch.tensor([3.0, -2.0, 0.0, 1.0, 6.0, -30.0, 0.5, 2.0])
+    qkv = torch.zeros(n_seqs, (heads + 2 * kv) * dim, dtype=dtype)
+    want = []
+    for s, (first, n) in enumerate(runs):
+        L = first + 1
+        keys, values = rnd(L, kv, dim, seed=1000 + s).to(dtype), rnd(L, kv, dim, seed=2000 + s).to(dtype)
+        q = rnd(1, heads, dim, seed=3000 + s, std=2.0).to(dtype)
+        fill_cache_by_pages(cache, table.cpu(), keys, values, page, s)
+        qkv[s, :heads * dim] = q.reshape(-1)
+        lo = first - first % chunk if chunk else 0
+        want.append(plain_attention(q, keys[lo:], values[lo:], [first - lo], scale, None, sinks))
+    got = k.paged_attention(qkv.to(dev), heads, kv, dim, scale, None, ctx, cache, chunk=chunk, sinks=sinks.to(dev))
+    close(got.view(n_seqs, heads, dim), torch.cat(want), "hip-bf16")
+    without = k.paged_attention(qkv.to(dev), heads, kv, dim, scale, None, ctx, cache, chunk=chunk)
+    ratio = (got.view(n_seqs, heads, dim).float().norm(dim=-1) / without.view(n_seqs, heads, dim).float().norm(dim=-1)).cpu()
+    assert float(ratio[:, 5].min()) > 0.999 and float(ratio[:, 4].max()) < 0.999   # a sink of -30 is nothing, one of 6 is felt
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("first,n", [(0, 2048), (0, 4096), (0, 9216), (7000, 1024), (100, 700)])
+@pytest.mark.parametrize("chunk", [None, 1500])
+def test_sinks_and_blocks_in_every_shape_of_prefill_workgroup(first, n, chunk):
+    """Long prompts and portions over a long past in bfloat16: the prefill kernel takes another shape of workgroup
+    by the number of row tiles (two sets of waves that share each pair of key tiles and merge at the end, or every
+    wave all tiles); the sink joins the denominator after that merge, and a block's first key bounds every tile
+    range.  The plain computation runs in float64 on the GPU."""
+    prefill_case(first, n, chunk, 16, 4, 64)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("first,n", [(0, 1300), (900, 300)])
+@pytest.mark.parametrize("dim", [144, 256])
+def test_sinks_and_blocks_in_prefill_with_large_heads(first, n, dim):
+    """Head sizes above 128 take workgroups of fewer tokens, and the largest load straight from the pages."""
+    prefill_case(first, n, 500, 4, 2, dim)
+
+
+def prefill_case(first, n, chunk, heads, kv, dim):
+    k, dev, dtype = setup("hip-bf16")
+    page, scale = 16, 0.09
+    L = first + n
+    ctx, table, n_pages, runs = step_context(dev, [(first, n)], page, k)
+    cache = empty_cache(dev, dtype, n_pages, kv, page, dim, dim, table)
+    keys, values = rnd(L, kv, dim, seed=500).to(dtype), rnd(L, kv, dim, seed=501).to(dtype)
+    q = rnd(n, heads, dim, seed=502, std=1.5).to(dtype)
+    fill_cache_by_pages(cache, table.cpu(), keys, values, page, 0)
+    sinks = (rnd(heads, seed=503, std=2.0) + 1.0)
+    qkv = torch.zeros(n, (heads + 2 * kv) * dim, dtype=dtype)
+    qkv[:, :heads * dim] = q.reshape(n, -1)
+    got = k.paged_attention(qkv.to(dev), heads, kv, dim, scale, None, ctx, cache, chunk=chunk, sinks=sinks.to(dev))
+    got = got.view(n, heads, dim).double()
+    qd, kd, vd = q.to(dev).double(), keys.to(dev).double(), values.to(dev).double()
+    qpos = torch.arange(first, L, device=dev)[:, None]
+    kpos = torch.arange(L, device=dev)[None, :]
+    seen = kpos <= qpos
+    if chunk:
+        seen &= (kpos // chunk) == (qpos // chunk)
+    worst = 0.0
+    for h in range(heads):
+        s = (qd[:, h] @ kd[:, h // (heads // kv)].T) * scale
+        s = s.masked_fill(~seen, float("-inf"))
+        want = plain.softmax_with_sink(s, sinks[h].double().to(dev)) @ vd[:, h // (heads // kv)]
+        worst = max(worst, float((got[:, h] - want).abs().max() / want.abs().max()))
+    assert worst <= TOL["hip-bf16"], worst
