@@ -25,6 +25,17 @@ def _feduzen_layer(ff, weights_of=None):
     return layer
 
 
+def _mogisun_layer(kind, moe):
+    if kind == "attention":
+        mixer = {"heads": 8, "kv_heads": 2, "dim": 64, "vdim": 64, "scale": 0.125, "q_temp": {"coef": 0.2, "every": 512}}
+    else:
+        mixer = {"heads": 8, "dim": 64, "vdim": 64, "tau": 8.0, "rank": 32}
+    mlp = {"kind": "dense", "ff": 1536}
+    if moe:
+        mlp = {"kind": "moe", "router": {"experts": 16, "top": 2}, "expert": {"ff": 384}, "shared": {"ff": 512}}
+    return {"type": kind, "mixer": mixer, "mlp": mlp}
+
+
 PRESETS = {
     "llama-3.2-3b": {
         "architectures": ["LlamaForCausalLM"], "model_type": "llama",
@@ -56,6 +67,14 @@ PRESETS = {
         "architecture": "Feduzen", "vocab": 4096, "width": 512, "embedding": {"scale": 2.0}, "norm": {"eps": 1e-6},
         "layers": [_feduzen_layer(1536), _feduzen_layer(None), _feduzen_layer(None, weights_of=1),
                    _feduzen_layer(1536), _feduzen_layer(1536, weights_of=0)],
+    },
+    # a small model of the Mogisun design: softmax and linear attention in turn, dense and routed feed-forwards, the
+    # middle four layers walked twice
+    "mogisun-small": {
+        "architecture": "Mogisun", "vocab": 4096, "width": 512, "norm": {"eps": 1e-6}, "logit_scale": 1.5,
+        "logit_softcap": 30.0, "loop": {"start": 1, "stop": 5, "times": 2},
+        "layers": [_mogisun_layer("attention", False), _mogisun_layer("gla", True), _mogisun_layer("attention", False),
+                   _mogisun_layer("gla", True), _mogisun_layer("attention", False), _mogisun_layer("gla", True)],
     },
     "tiny-a": {
         "architectures": ["LlamaForCausalLM"], "model_type": "llama",

@@ -8,6 +8,7 @@
 //   x += bias                                                     (if bias is given)
 //   x  = x * rsqrt(mean(x^2) + eps) * gain                         (if gains are given; one gain of head_dim for
 //                                                                   all q heads, one for all k heads)
+//   x *= 1 + coef * ln(floor((pos + 1) / every) + 1)               (q heads only, if a query temperature is given)
 //   (x_i, x_{i+r/2}) <- (x_i c_i - x_{i+r/2} s_i, x_{i+r/2} c_i + x_i s_i),  i < r/2, r = rotary_dim,
 //                       c, s from the float tables at the token's absolute position; elements from r on pass
 //
@@ -32,6 +33,12 @@
 #define QKP_MAX_HEAD_DIM 256
 #define QKP_WAVES 4
 #define QKP_PER_LANE (QKP_MAX_HEAD_DIM / SIA_WAVE)
+
+// A query's temperature: 1 + coef * ln(floor((pos + 1) / every) + 1), a step function of the position that sharpens
+// the scores of late queries (every <= 0: none).
+__device__ __forceinline__ float query_temperature(int pos, float coef, int every) {
+    return 1.f + coef * logf((float)((pos + 1) / every + 1));
+}
 
 template <typename T>
 __device__ __forceinline__ void write_values(const T* __restrict__ qkv, int row_stride, const float* __restrict__ bias,
@@ -85,7 +92,8 @@ __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_kernel(
     const float* __restrict__ sin_table, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
     const int* __restrict__ block_table, int table_width, T* __restrict__ k_pages, T* __restrict__ v_pages,
     int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim, int rotary_dim, int page_size, int v_group,
-    int k_row, int v_rows, T* q_out, int q_row_stride, int q_head_stride) {   // q_out may be qkv
+    int k_row, int v_rows, T* q_out, int q_row_stride, int q_head_stride, float temp_coef,
+    int temp_every) {   // q_out may be qkv
     const int n = blockIdx.x, wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE;
     const int pos = positions[n];
     const int half = rotary_dim / 2;
@@ -129,6 +137,11 @@ __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_kernel(
             if (d < head_dim) x[j] = x[j] * inv * gain[d];
         }
     }
+    if (is_q && temp_every > 0) {
+        const float temp = query_temperature(pos, temp_coef, temp_every);
+#pragma unroll
+        for (int j = 0; j < QKP_PER_LANE; ++j) x[j] *= temp;
+    }
     T* dst = is_q ? q_out + (size_t)n * q_row_stride + h * q_head_stride
                   : (page >= 0 ? k_pages + (((size_t)page * n_kv + h) * page_size + off) * k_row : nullptr);
 #pragma unroll
@@ -163,7 +176,8 @@ __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_vec_kernel(
     const float* __restrict__ sin_table, const int* __restrict__ positions, const int* __restrict__ seq_of_token,
     const int* __restrict__ block_table, int table_width, T* __restrict__ k_pages, T* __restrict__ v_pages,
     int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim, int rotary_dim, int page_size, int v_group,
-    int k_row, int v_rows, T* q_out, int q_row_stride, int q_head_stride) {   // q_out may be qkv
+    int k_row, int v_rows, T* q_out, int q_row_stride, int q_head_stride, float temp_coef,
+    int temp_every) {   // q_out may be qkv
     const int n = blockIdx.x, wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE;
     const int pos = positions[n];
     const int half = rotary_dim / 2;
@@ -216,6 +230,11 @@ __global__ __launch_bounds__(QKP_WAVES* SIA_WAVE) void qk_prepare_vec_kernel(
 #pragma unroll
         for (int i = 0; i < 8; ++i) x[i] = x[i] * inv * g[i];
     }
+    if (is_q && temp_every > 0) {
+        const float temp = query_temperature(pos, temp_coef, temp_every);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) x[i] *= temp;
+    }
     if (rotary_dim > 0) {   // wave-uniform: every lane takes the exchange
         const int mate = turns ? (low ? lane + half / 8 : lane - half / 8) : lane;
         float other[8];
@@ -241,7 +260,7 @@ SIA_EXPORT int sia_qk_prepare(void* qkv, int row_stride, const float* bias, cons
                               const int* seq_of_token, const int* block_table, int table_width, void* k_pages,
                               void* v_pages, int n_tokens, int n_heads, int n_kv, int head_dim, int value_dim,
                               int rotary_dim, int page_size, int k_row, int v_rows, void* q_out, int q_row_stride,
-                              int q_head_stride, int dtype, hipStream_t stream) {
+                              int q_head_stride, float temp_coef, int temp_every, int dtype, hipStream_t stream) {
     if (n_tokens <= 0) return 0;
     if (head_dim <= 0 || head_dim > QKP_MAX_HEAD_DIM || value_dim <= 0 || n_heads < 0 || n_kv < 0) return SIA_BAD_ARGUMENT;
     if (rotary_dim < 0 || rotary_dim > head_dim || (rotary_dim & 1)) return SIA_BAD_ARGUMENT;
@@ -270,12 +289,14 @@ SIA_EXPORT int sia_qk_prepare(void* qkv, int row_stride, const float* bias, cons
             hipLaunchKernelGGL(qk_prepare_vec_kernel<T>, grid, block, 0, stream, (T*)qkv, row_stride, bias, q_gain,  \
                                k_gain, eps, cos_table, sin_table, positions, seq_of_token, block_table, table_width, \
                                (T*)k_pages, (T*)v_pages, n_tokens, n_heads, n_kv, head_dim, value_dim, rotary_dim,   \
-                               page_size, v_group, k_row, v_rows, (T*)q_out, q_row_stride, q_head_stride);           \
+                               page_size, v_group, k_row, v_rows, (T*)q_out, q_row_stride, q_head_stride, temp_coef,  \
+                               temp_every);                                                                          \
         else                                                                                                         \
             hipLaunchKernelGGL(qk_prepare_kernel<T>, grid, block, 0, stream, (T*)qkv, row_stride, bias, q_gain,      \
                                k_gain, eps, cos_table, sin_table, positions, seq_of_token, block_table, table_width, \
                                (T*)k_pages, (T*)v_pages, n_tokens, n_heads, n_kv, head_dim, value_dim, rotary_dim,   \
-                               page_size, v_group, k_row, v_rows, (T*)q_out, q_row_stride, q_head_stride);           \
+                               page_size, v_group, k_row, v_rows, (T*)q_out, q_row_stride, q_head_stride, temp_coef,  \
+                               temp_every);                                                                          \
     } while (0)
     if (dtype == SIA_F32) LAUNCH(float);
     else if (dtype == SIA_BF16) LAUNCH(bf16_t);

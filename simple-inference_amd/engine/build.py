@@ -46,6 +46,8 @@ def count_parameters(model, model_cfg) -> int:
         n = 1
         for d in spec.shape:
             n *= d
+        if n < 0:       # a size that only the checkpoint gives: nothing to count before the weights are bound
+            return -1
         total += n
     formula = getattr(model_cfg, "num_parameters", None)
     if formula is not None and formula() != total:

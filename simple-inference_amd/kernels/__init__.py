@@ -32,8 +32,22 @@ _SIGNATURES = {
     "sia_activation": [_c_ptr, _c_ptr, _c_ll, _c_int, _c_int, _c_ptr],
     "sia_qk_prepare": [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
                        _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr,
-                       _c_int, _c_int, _c_int, _c_ptr],
+                       _c_int, _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "sia_qk_prepare_max_head_dim": [],
+    "sia_gated_add_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+                              _c_float, _c_int, _c_ptr],
+    "sia_add_bias": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_head_gate": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_side_by_side": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_scale_softcap": [_c_ptr, _c_ll, _c_float, _c_float, _c_ptr],
+    "sia_gla_max_dims": [],
+    "sia_gla_recurrent": [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                          _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float,
+                          _c_int, _c_ptr],
+    "sia_moe_route": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_moe_gate_up": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_moe_down": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+                     _c_int, _c_ptr],
     "sia_gemm_skinny_act": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_add_rmsnorm": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "sia_swiglu": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
@@ -319,12 +333,20 @@ class HipKernels:
         return residual if lowered is None else lowered
 
     # -- residual add + rms norm ---------------------------------------------
-    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None):
+    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None, gate=None, gate_bias=None,
+                    delta_bias=None):
+        """``residual += delta`` and the RMS norm of the sum.  With ``gate`` (the logits of an elementwise gate:
+        ``[n, hidden]``, which may be columns of a wider matrix) the sum is
+        ``residual += (delta + delta_bias) * sigmoid(gate + gate_bias)``."""
         n, hidden = residual.shape
         self._want(residual, "residual", torch.float32)
         self._want(weight, "norm weight", torch.float32, (hidden,))
         if out_dtype not in _DT:
             raise KernelError(f"norm output dtype {out_dtype} is not float32 or bfloat16")
+        if gate is not None:
+            return self._gated_add(residual, delta, gate, gate_bias, delta_bias, weight, eps, out_dtype, rows)
+        if gate_bias is not None or delta_bias is not None:
+            raise KernelError("a bias of the gate or of the delta comes with a gate only")
         if delta is not None:
             self._want(delta, "delta", out_dtype, (n, hidden))
         n_out = n
@@ -335,6 +357,168 @@ class HipKernels:
         self._check(self.core.sia_add_rmsnorm(_ptr(residual), _ptr(delta), _ptr(weight), _ptr(out), _ptr(rows),
                                               n_out, hidden, float(eps), _DT[out_dtype], self._stream()),
                     "add_rmsnorm")
+        return out
+
+    def gated_add(self, residual, delta, gate=None, gate_bias=None, delta_bias=None):
+        """``residual += (delta + delta_bias) * sigmoid(gate + gate_bias)`` and nothing else (without ``gate`` the
+        factor is 1)."""
+        self._want(residual, "residual", torch.float32)
+        self._gated_add(residual, delta, gate, gate_bias, delta_bias, None, 0.0, delta.dtype, None)
+
+    def _columns(self, t, what, dtype, shape):
+        """Row stride of a matrix that may be a run of columns of a wider one (elements of a row contiguous)."""
+        if t.device.type != "cuda" or t.dtype != dtype or t.dim() != 2 or tuple(t.shape) != tuple(shape):
+            raise KernelError(f"{what} must be {dtype} {tuple(shape)} on the GPU, is {t.dtype} {tuple(t.shape)} on {t.device}")
+        if t.shape[1] > 1 and t.stride(1) != 1:
+            raise KernelError(f"the elements of a row of {what} must be contiguous")
+        return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+    def _gated_add(self, residual, delta, gate, gate_bias, delta_bias, weight, eps, out_dtype, rows):
+        n, hidden = residual.shape
+        self._want(delta, "delta", out_dtype, (n, hidden))
+        stride = self._columns(gate, "gate logits", out_dtype, (n, hidden)) if gate is not None else 0
+        for t, what in ((gate_bias, "gate bias"), (delta_bias, "delta bias")):
+            if t is not None:
+                self._want(t, what, torch.float32, (hidden,))
+        n_out, out = n, None
+        if rows is not None:
+            self._want(rows, "rows", torch.int32)
+            n_out = rows.numel()
+        if weight is not None:
+            out = torch.empty((n_out, hidden), dtype=out_dtype, device=residual.device)
+        self._check(self.core.sia_gated_add_rmsnorm(_ptr(residual), _ptr(delta), _ptr(delta_bias), _ptr(gate), stride,
+                                                    _ptr(gate_bias), _ptr(weight), _ptr(out), _ptr(rows), n_out, hidden,
+                                                    float(eps), _DT[out_dtype], self._stream()), "gated_add_rmsnorm")
+        return out
+
+    def add_bias(self, y, bias):
+        """``y += bias`` over the rows, in place."""
+        self._want(y, "rows")
+        if y.dtype not in _DT or y.dim() != 2:
+            raise KernelError(f"add_bias takes a float32 or bfloat16 matrix, got {y.dtype} {tuple(y.shape)}")
+        self._want(bias, "bias", torch.float32, (y.shape[1],))
+        self._check(self.core.sia_add_bias(_ptr(y), _ptr(bias), y.shape[0], y.shape[1], _DT[y.dtype], self._stream()),
+                    "add_bias")
+        return y
+
+    def head_gate(self, out, logits, n_heads):
+        """``out[n, h, :] *= sigmoid(logits[n, h])`` in place; ``logits`` may be columns of a wider matrix."""
+        self._want(out, "attention output")
+        n, width = out.shape
+        if out.dtype not in _DT or width % n_heads:
+            raise KernelError(f"head gate takes float32 or bfloat16 rows of {n_heads} heads, got {out.dtype} {tuple(out.shape)}")
+        stride = self._columns(logits, "head gate logits", out.dtype, (n, n_heads))
+        self._check(self.core.sia_head_gate(_ptr(out), _ptr(logits), stride, n, n_heads, width // n_heads,
+                                            _DT[out.dtype], self._stream()), "head_gate")
+        return out
+
+    def side_by_side(self, a, b, dtype):
+        """``[a, b]`` along the columns, lowered to ``dtype``: two float streams as the input of one product."""
+        self._want(a, "first stream", torch.float32)
+        self._want(b, "second stream", torch.float32, tuple(a.shape))
+        if dtype not in _DT or a.dim() != 2:
+            raise KernelError(f"side_by_side makes float32 or bfloat16 rows of two matrices, got {dtype} of {tuple(a.shape)}")
+        out = torch.empty((a.shape[0], 2 * a.shape[1]), dtype=dtype, device=a.device)
+        self._check(self.core.sia_side_by_side(_ptr(a), _ptr(b), _ptr(out), a.shape[0], a.shape[1], _DT[dtype],
+                                               self._stream()), "side_by_side")
+        return out
+
+    def scale_softcap(self, logits, scale=1.0, cap=None):
+        """``logits * scale`` and then, with ``cap``, ``cap * tanh(. / cap)``: in place, float."""
+        self._want(logits, "logits", torch.float32)
+        if cap is not None and not cap > 0:
+            raise KernelError(f"a soft cap must be positive, got {cap}")
+        self._check(self.core.sia_scale_softcap(_ptr(logits), logits.numel(), float(scale), float(cap or 0.0),
+                                                self._stream()), "scale_softcap")
+        return logits
+
+    # -- linear attention with a state ---------------------------------------------
+    def gla_recurrent(self, proj, columns, a2, a2_bias, norm_weight, n_heads, key_dim, value_dim, tau, q_scale, eps,
+                      ctx, cache):
+        """Gated linear attention over the step's runs of tokens, from the projected rows ``proj`` whose column
+        offsets ``columns = (q, k, v, g, a)`` name the queries and keys ``[n_heads * key_dim]``, the values and output
+        gates ``[n_heads * value_dim]`` and the low-rank decay input ``[rank]``; ``a2 [n_heads * key_dim, rank]``.
+        The state ``cache.state [slots, n_heads, key_dim, value_dim]`` (float) is read and left updated.  Returns
+        the normed and gated output ``[tokens, n_heads * value_dim]``."""
+        self._want(proj, "projected rows")
+        n, width = proj.shape
+        if proj.dtype not in _DT or n != ctx.n_tokens:
+            raise KernelError(f"projected rows {proj.dtype} {tuple(proj.shape)} do not fit a step of {ctx.n_tokens} tokens")
+        rank = a2.shape[1]
+        self._want(a2, "decay matrix", proj.dtype, (n_heads * key_dim, rank))
+        if a2_bias is not None:
+            self._want(a2_bias, "decay bias", torch.float32, (n_heads * key_dim,))
+        self._want(norm_weight, "output norm weight", torch.float32, (value_dim,))
+        q, k, v, g, a = (int(c) for c in columns)
+        for first, size, what in ((q, n_heads * key_dim, "q"), (k, n_heads * key_dim, "k"), (v, n_heads * value_dim, "v"),
+                                  (g, n_heads * value_dim, "g"), (a, rank, "decay input")):
+            if first < 0 or first + size > width:
+                raise KernelError(f"columns {first} .. {first + size} of {what} lie outside a row of {width}")
+        state = cache.state
+        if state is None:
+            raise KernelError("gated linear attention needs its state rows")
+        self._want(state, "state", torch.float32)
+        if tuple(state.shape[1:]) != (n_heads, key_dim, value_dim):
+            raise KernelError(f"state rows {tuple(state.shape[1:])} are not [{n_heads}, {key_dim}, {value_dim}]")
+        limit = self.core.sia_gla_max_dims()
+        if not (0 < key_dim <= limit and 0 < value_dim <= limit):
+            raise KernelError(f"head sizes {key_dim} x {value_dim} are outside what the kernel takes (up to {limit})")
+        out = torch.empty((n, n_heads * value_dim), dtype=proj.dtype, device=proj.device)
+        self._check(self.core.sia_gla_recurrent(
+            _ptr(proj), width, q, k, v, g, a, _ptr(a2), _ptr(a2_bias), _ptr(norm_weight), _ptr(state), _ptr(ctx.cu_q),
+            _ptr(ctx.state_slots), _ptr(out), ctx.n_seqs, ctx.max_q_len, n_heads, key_dim, value_dim, rank, float(tau),
+            float(q_scale), float(eps), _DT[proj.dtype], self._stream()), "gla_recurrent")
+        return out
+
+    def check_recurrent_geometry(self, key_dim: int, value_dim: int) -> None:
+        limit = self.core.sia_gla_max_dims()
+        if not (0 < key_dim <= limit and 0 < value_dim <= limit):
+            raise KernelError(f"head sizes {key_dim} x {value_dim} are outside what the recurrent kernel takes (up to {limit})")
+
+    # -- mixture of experts ------------------------------------------------------------
+    def moe_route(self, h, router, top):
+        """The ``top`` experts of every row with the largest router logits ``h @ router^T`` (float; ties go to the
+        lower index) and the softmax over their logits alone: ``(ids [n, top] int32, weights [n, top] float32)``."""
+        self._want(h, "router input")
+        n, width = h.shape
+        experts = router.shape[0]
+        self._want(router, "router", torch.float32, (experts, width))
+        if h.dtype not in _DT:
+            raise KernelError(f"router input must be float32 or bfloat16, is {h.dtype}")
+        ids = torch.empty((n, top), dtype=torch.int32, device=h.device)
+        weights = torch.empty((n, top), dtype=torch.float32, device=h.device)
+        self._check(self.core.sia_moe_route(_ptr(h), _ptr(router), _ptr(ids), _ptr(weights), n, width, experts, int(top),
+                                            _DT[h.dtype], self._stream()), "moe_route")
+        return ids, weights
+
+    def moe_experts(self, h, w_gate_up, w_down, ids, weights, shared=None, shared_gate=None):
+        """``sum_k weights[n, k] * expert_{ids[n, k]}(h[n])`` with ``expert_e(x) = W2_e (silu(Wg_e x) * (Wu_e x))``,
+        ``w_gate_up [E, 2 ff, width]`` (gate rows first), ``w_down [E, width, ff]``; plus ``shared`` ``[n, width]``
+        (times ``sigmoid(shared_gate [n, 1])`` if given), the sum rounded once."""
+        self._want(h, "expert input")
+        n, width = h.shape
+        experts, two_ff, _ = w_gate_up.shape
+        ff, top = two_ff // 2, ids.shape[1]
+        self._want(w_gate_up, "expert gate/up weights", h.dtype, (experts, 2 * ff, width))
+        self._want(w_down, "expert down weights", h.dtype, (experts, width, ff))
+        self._want(ids, "expert ids", torch.int32, (n, top))
+        self._want(weights, "expert weights", torch.float32, (n, top))
+        if h.dtype not in _DT:
+            raise KernelError(f"expert input must be float32 or bfloat16, is {h.dtype}")
+        gate_stride = 0
+        if shared is not None:
+            self._want(shared, "shared expert output", h.dtype, (n, width))
+            if shared_gate is not None:
+                gate_stride = self._columns(shared_gate, "shared expert gate", h.dtype, (n, 1))
+        elif shared_gate is not None:
+            raise KernelError("a shared expert's gate comes with its output")
+        act = torch.empty((n * top, ff), dtype=h.dtype, device=h.device)
+        out = torch.empty((n, width), dtype=h.dtype, device=h.device)
+        self._check(self.core.sia_moe_gate_up(_ptr(h), _ptr(w_gate_up), _ptr(ids), _ptr(act), n, width, ff, top,
+                                              _DT[h.dtype], self._stream()), "moe_gate_up")
+        self._check(self.core.sia_moe_down(_ptr(act), _ptr(w_down), _ptr(ids), _ptr(weights), _ptr(shared),
+                                           _ptr(shared_gate), gate_stride, _ptr(out), n, width, ff, top, _DT[h.dtype],
+                                           self._stream()), "moe_down")
         return out
 
     # -- matrix product --------------------------------------------------------
@@ -566,7 +750,7 @@ class HipKernels:
             "rope_kv_write")
 
     def qkv_to_cache(self, x, w_qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache,
-                     value_dim=None, bias=None, qk_norm=None, page_dim=None):
+                     value_dim=None, bias=None, qk_norm=None, page_dim=None, q_temp=None, extra_columns=0):
         """The q/k/v product, the rotation of q and k and the write of k and v into the pages.  Returns the
         ``[tokens, (n_heads + 2 n_kv_written) head_dim]`` matrix whose q columns hold the rotated queries; its
         k and v columns are not to be read (for few rows one kernel does all three and never writes them).
@@ -577,9 +761,14 @@ class HipKernels:
 
         ``page_dim`` (see ``attention_page_dim``): the pages' keys and values are both that wide; the result is then
         ``[tokens, n_heads * page_dim]``, the queries with zeros behind every head, and attention is called with
-        ``page_dim`` for the head size."""
+        ``page_dim`` for the head size.
+
+        ``q_temp``: ``(coef, every)``, every query is multiplied by ``1 + coef * ln(floor((pos + 1) / every) + 1)``
+        after its norm.  ``extra_columns``: the weight has that many further rows behind v, whose products are only
+        carried along; the result is then the pair (that matrix, the further columns of the projected rows)."""
         M, K = x.shape
-        if value_dim is not None or bias is not None or qk_norm is not None or page_dim is not None:
+        if (value_dim is not None or bias is not None or qk_norm is not None or page_dim is not None
+                or q_temp is not None or extra_columns):
             qkv = self.linear(x, w_qkv)
             q_out = None
             if page_dim is not None:
@@ -593,8 +782,11 @@ class HipKernels:
                 if q_out is None:
                     q_out = kept[key] = torch.zeros((M, n_heads * page_dim), dtype=qkv.dtype, device=qkv.device)
             self.qk_prepare(qkv, n_heads, n_kv_written, head_dim, value_dim or head_dim, rotary_dim, cos, sin, bias,
-                            qk_norm, ctx, cache, page_dim, q_out)
-            return qkv if q_out is None else q_out
+                            qk_norm, ctx, cache, page_dim, q_out, q_temp, extra_columns)
+            queries = qkv if q_out is None else q_out
+            if extra_columns:
+                return queries, qkv[:, qkv.shape[1] - extra_columns:]
+            return queries
         if (self.use_skinny_gemm and self.fuse_rope and n_kv_written and x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16
                 and M <= self._skinny_rows and rotary_dim == head_dim and head_dim % 2 == 0 and K % 64 == 0):
             x, partials, n_partials, norm_eps = self._scaled(x)
@@ -638,7 +830,7 @@ class HipKernels:
         return wide
 
     def qk_prepare(self, qkv, n_heads, n_kv_written, head_dim, value_dim, rotary_dim, cos, sin, bias, qk_norm, ctx,
-                   cache, page_dim=None, q_out=None):
+                   cache, page_dim=None, q_out=None, q_temp=None, extra_columns=0):
         """Bias, per-head RMS norm of q and k, rotation, and the write of k and v into the pages, on the projected
         rows ``[q heads | k heads | v heads]`` (q and k heads ``head_dim`` wide, v heads ``value_dim``); q is left in
         place."""
@@ -646,9 +838,10 @@ class HipKernels:
         n, width = qkv.shape
         if qkv.dtype not in _DT:
             raise KernelError(f"qkv must be float32 or bfloat16, is {qkv.dtype}")
-        if width != n_heads * head_dim + n_kv_written * (head_dim + value_dim):
+        own = n_heads * head_dim + n_kv_written * (head_dim + value_dim)
+        if width != own + extra_columns:
             raise KernelError(f"qkv row of {width} does not hold {n_heads} q heads and {n_kv_written} k heads of "
-                              f"{head_dim} and as many v heads of {value_dim}")
+                              f"{head_dim}, as many v heads of {value_dim} and {extra_columns} further columns")
         if n != ctx.n_tokens:
             raise KernelError(f"qkv has {n} rows, the step {ctx.n_tokens} tokens")
         if not 0 < head_dim <= self.core.sia_qk_prepare_max_head_dim():
@@ -660,7 +853,10 @@ class HipKernels:
                     raise KernelError(f"{what} {tuple(t.shape)} does not cover position {ctx.max_kv_len - 1} "
                                       f"with {rotary_dim // 2} pairs")
         if bias is not None:
-            self._want(bias, "q/k/v bias", torch.float32, (width,))
+            self._want(bias, "q/k/v bias", torch.float32, (own,))
+        temp_coef, temp_every = (float(q_temp[0]), int(q_temp[1])) if q_temp is not None else (0.0, 0)
+        if q_temp is not None and temp_every <= 0:
+            raise KernelError(f"a query temperature steps every so many positions, got {temp_every}")
         q_gain = k_gain = None
         eps = 0.0
         if qk_norm is not None:
@@ -683,7 +879,7 @@ class HipKernels:
             _ptr(cos) if rotary_dim else None, _ptr(sin) if rotary_dim else None, _ptr(ctx.positions),
             _ptr(ctx.seq_of_token), _ptr(table), table.shape[1] if table is not None else 0, _ptr(k_pages),
             _ptr(v_pages), n, n_heads, n_kv_written, head_dim, value_dim, rotary_dim, page_size, k_row, v_rows,
-            _ptr(q_out), n_heads * page_dim if page_dim else 0, page_dim or 0, _DT[qkv.dtype],
+            _ptr(q_out), n_heads * page_dim if page_dim else 0, page_dim or 0, temp_coef, temp_every, _DT[qkv.dtype],
             self._stream()), "qk_prepare")
 
     def _check_pages(self, k_pages, v_pages, table, page_size, n_kv, head_dim, dtype, ctx, value_dim=None):

@@ -1,2 +1,3 @@
 from . import llama  # noqa: F401  (registers LlamaForCausalLM)
 from . import feduzen  # noqa: F401  (registers Feduzen)
+from . import mogisun  # noqa: F401  (registers Mogisun)

@@ -1,17 +1,17 @@
 from .plan import LayerSpec, ModelPlan, PagedKVNeed, PartSpec, StateNeed, TensorSpec
 from .registry import (
-    BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSITION_ENCODINGS,
-    register_block, register_embedding, register_feed_forward, register_head, register_mixer, register_norm,
-    register_position_encoding,
+    BLOCKS, EMBEDDINGS, FEED_FORWARDS, GATES, HEADS, MIXERS, NORMS, POSITION_ENCODINGS, STREAM_OPS,
+    register_block, register_embedding, register_feed_forward, register_gate, register_head, register_mixer,
+    register_norm, register_position_encoding, register_stream_op,
 )
-from .context import BuildEnv, LayerCache, ResidualStream, StepContext
-from . import norm, rope, attention, swiglu, dense, block, embedding  # noqa: F401  (registers the built-in kinds)
+from .context import BiasedDelta, BuildEnv, LayerCache, ResidualStream, StepContext
+from . import norm, rope, attention, swiglu, dense, block, embedding, gate, stream_ops, gla, moe  # noqa: F401  (registers the built-in kinds)
 from .model import DecoderModel
 
 __all__ = [
     "LayerSpec", "ModelPlan", "PagedKVNeed", "PartSpec", "StateNeed", "TensorSpec",
-    "BLOCKS", "EMBEDDINGS", "FEED_FORWARDS", "HEADS", "MIXERS", "NORMS", "POSITION_ENCODINGS",
-    "register_block", "register_embedding", "register_feed_forward", "register_head", "register_mixer",
-    "register_norm", "register_position_encoding",
-    "BuildEnv", "LayerCache", "ResidualStream", "StepContext", "DecoderModel",
+    "BLOCKS", "EMBEDDINGS", "FEED_FORWARDS", "GATES", "HEADS", "MIXERS", "NORMS", "POSITION_ENCODINGS", "STREAM_OPS",
+    "register_block", "register_embedding", "register_feed_forward", "register_gate", "register_head", "register_mixer",
+    "register_norm", "register_position_encoding", "register_stream_op",
+    "BiasedDelta", "BuildEnv", "LayerCache", "ResidualStream", "StepContext", "DecoderModel",
 ]

@@ -27,12 +27,20 @@ Further forms, each switched on by a parameter of its own and free to combine:
 * ``sink``: a learned logit per query head that competes in the softmax but carries no value: the weights of
   the real keys are ``exp(s_j) / (sum_i exp(s_i) + exp(sink_h))``, with ``sink_h`` taken as it is (``scale``
   applies to the dot products only).
+* ``qk_norm`` with ``"gain": False``: the same division by the root mean square without learned gains.
+* ``q_temp`` (``{"coef": c, "every": n}``): a query at position ``p`` is multiplied by
+  ``1 + c * ln(floor((p + 1) / n) + 1)`` after its norm, so late queries score more sharply.
+* ``out_gate``: head ``h``'s output is multiplied by ``sigmoid((G x)_h)``, one number per token and head, ``G
+  [Hq, H]`` reading the mixer's own input; its rows ride at the end of the stacked projection.
+* ``o_bias``: the output projection has a bias; it is handed on with the result (``BiasedDelta``) so that the sum
+  into the residual can take it in passing.
 """
 
 from __future__ import annotations
 
 import torch
 
+from .context import BiasedDelta
 from .plan import PagedKVNeed, TensorSpec
 from .registry import POSITION_ENCODINGS, register_mixer
 
@@ -50,7 +58,7 @@ def _shared_position_encoding(spec, env):
 class Attention:
     """params: hidden_size, num_heads, num_kv_heads, head_dim, position
     (``{"kind", "params"}``), and optionally window, scale, kv_from_layer, value_head_dim, bias, qk_norm, chunk,
-    sink."""
+    sink, q_temp, out_gate, o_bias."""
 
     def __init__(self, params, env):
         self.hidden = int(params["hidden_size"])
@@ -71,13 +79,21 @@ class Attention:
         self.bias = bool(params.get("bias", False))
         qk_norm = params.get("qk_norm")
         self.qk_norm_eps = float(qk_norm["eps"]) if qk_norm else None
+        self.qk_norm_gain = bool(qk_norm.get("gain", True)) if qk_norm else False
+        q_temp = params.get("q_temp")
+        self.q_temp = (float(q_temp["coef"]), int(q_temp["every"])) if q_temp else None
+        if self.q_temp is not None and self.q_temp[1] <= 0:
+            raise ValueError(f"q_temp.every must be positive, got {self.q_temp[1]}")
+        self.out_gate = bool(params.get("out_gate", False))
+        self.o_bias = bool(params.get("o_bias", False))
         self.chunk = params.get("chunk")
         if self.chunk is not None:
             self.chunk = int(self.chunk)
             if self.chunk <= 0:
                 raise ValueError(f"chunk must be positive, got {self.chunk}")
         self.sink = bool(params.get("sink", False))
-        if self.kv_from_layer is not None and (self.bias or self.qk_norm_eps is not None or self.value_dim != self.head_dim):
+        if self.kv_from_layer is not None and (self.bias or self.qk_norm_eps is not None or self.value_dim != self.head_dim
+                                               or self.out_gate or self.q_temp is not None):
             raise ValueError("a mixer that reads another layer's keys and values has plain q heads of the keys' width")
         self.position = _shared_position_encoding(params.get("position", {"kind": "none", "params": {}}), env)
         if self.position.rotary_dim > self.head_dim:
@@ -91,7 +107,8 @@ class Attention:
         self.env = env
         self.w_qkv = None
         self.w_o = None
-        self.b_qkv = self.q_gain = self.k_gain = self.sinks = None
+        self.b_qkv = self.q_gain = self.k_gain = self.sinks = self.b_o = None
+        self.gate_columns = 0
 
     takes_scaled_rows = True   # the input goes to ``qkv_to_cache`` only
 
@@ -110,17 +127,23 @@ class Attention:
         if self.bias:
             specs.update({"q_bias": TensorSpec((q,), "vector"), "k_bias": TensorSpec((kv,), "vector"),
                           "v_bias": TensorSpec((v,), "vector")})
-        if self.qk_norm_eps is not None:
+        if self.qk_norm_eps is not None and self.qk_norm_gain:
             specs.update({"q_norm": TensorSpec((self.head_dim,), "vector"), "k_norm": TensorSpec((self.head_dim,), "vector")})
         if self.sink:
             specs["sink"] = TensorSpec((self.num_heads,), "vector")
+        if self.out_gate:
+            specs["gate"] = TensorSpec((self.num_heads, self.hidden))
+        if self.o_bias:
+            specs["o_bias"] = TensorSpec((self.hidden,), "vector")
         return specs
 
     def bind(self, tensors):
-        if self.writes_kv:
-            self.w_qkv = torch.cat([tensors["q"], tensors["k"], tensors["v"]], dim=0).contiguous()
-        else:
-            self.w_qkv = tensors["q"].contiguous()
+        stacked = [tensors["q"], tensors["k"], tensors["v"]] if self.writes_kv else [tensors["q"]]
+        if self.out_gate:   # the gate's rows behind v, filled up with zero rows so that a projected row stays aligned
+            self.gate_columns = -(-self.num_heads // 8) * 8
+            g = tensors["gate"]
+            stacked += [g, g.new_zeros((self.gate_columns - self.num_heads, self.hidden))]
+        self.w_qkv = torch.cat(stacked, dim=0).contiguous()
         self.w_o = tensors["o"].contiguous()
         if self.page_dim is not None:   # the attention's rows come with page_dim elements a head: zero columns for the rest
             wide = self.w_o.new_zeros((self.hidden, self.num_heads, self.page_dim))
@@ -128,8 +151,12 @@ class Attention:
             self.w_o = wide.view(self.hidden, self.num_heads * self.page_dim)
         if self.bias:
             self.b_qkv = torch.cat([tensors["q_bias"], tensors["k_bias"], tensors["v_bias"]]).contiguous()
-        if self.qk_norm_eps is not None:
+        if self.qk_norm_eps is not None and self.qk_norm_gain:
             self.q_gain, self.k_gain = tensors["q_norm"].contiguous(), tensors["k_norm"].contiguous()
+        elif self.qk_norm_eps is not None:
+            self.q_gain = self.k_gain = torch.ones(self.head_dim, dtype=torch.float32, device=self.w_qkv.device)
+        if self.o_bias:
+            self.b_o = tensors["o_bias"].contiguous()
         if self.sink:
             self.sinks = tensors["sink"].contiguous()
         prepare = getattr(self.env.kernels, "prepare_pending_weight", None)
@@ -150,7 +177,7 @@ class Attention:
     def _options(self) -> bool:
         """Whether any of the further forms is switched on (the kernels then get them as keyword arguments)."""
         return (self.bias or self.qk_norm_eps is not None or self.sink or self.chunk is not None
-                or self.value_dim != self.head_dim)
+                or self.value_dim != self.head_dim or self.q_temp is not None or self.out_gate)
 
     def cache_need(self):
         if self.page_dim is not None:
@@ -180,10 +207,21 @@ class Attention:
                 attend["chunk"] = self.chunk
             if self.sink:
                 attend["sinks"] = self.sinks
+            if self.q_temp is not None:
+                project["q_temp"] = self.q_temp
+            if self.out_gate:
+                project["extra_columns"] = self.gate_columns
         qkv = k.qkv_to_cache(
             h, self.w_qkv, self.num_heads, self.num_kv_heads if self.writes_kv else 0, self.head_dim,
             self.position.rotary_dim, cos, sin, ctx, cache, **project)
+        gate_logits = None
+        if self.out_gate:
+            qkv, further = qkv
+            gate_logits = further[:, :self.num_heads]
         out = k.paged_attention(
             qkv, self.num_heads, self.num_kv_heads, self.page_dim or self.head_dim, self.scale, self.window, ctx, cache,
             **attend)
-        return k.pending_linear(out, self.w_o)   # the norm after it may have it added into the residual
+        if gate_logits is not None:
+            out = k.head_gate(out, gate_logits, self.num_heads)
+        y = k.pending_linear(out, self.w_o)   # the norm after it may have it added into the residual
+        return BiasedDelta(y, self.b_o, k) if self.o_bias else y

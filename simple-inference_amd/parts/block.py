@@ -9,6 +9,11 @@ Output-norm: ``x += norm1(mixer(x))``; ``x += norm2(feed_forward(x))``.  Mixer a
 un-normed stream as input (rounded to the compute dtype), and each norm is applied to its sublayer's result; the kernel that adds the normed
 output into the float32 residual also leaves the rounded residual for the next sublayer.  A layer of this kind
 may have no feed-forward.
+
+Gated pre-norm: ``h = norm1(x); x += sigmoid(G1 h + g1) * mixer(h)``, then the same with the feed-forward if the
+layer has one.  Each sublayer's result passes an elementwise gate computed from the sublayer's own input; the gate's
+logits travel with the pending delta (``stream.gate``) and the sigmoid, the product and the sum happen inside the
+kernel of the norm that follows.
 """
 
 from __future__ import annotations
@@ -76,3 +81,23 @@ class OutputNormBlock:
         x = self.mixer_norm.add_normed(stream, self.mixer.forward(x, ctx, cache))
         if self.feed_forward is not None:
             self.feed_forward_norm.add_normed(stream, self.feed_forward.forward(x, ctx))
+
+
+@register_block("gated_prenorm")
+class GatedPreNormBlock:
+    def __init__(self, mixer, mixer_norm, mixer_gate, feed_forward=None, feed_forward_norm=None, feed_forward_gate=None):
+        if not ((feed_forward is None) == (feed_forward_norm is None) == (feed_forward_gate is None)):
+            raise ValueError("a gated pre-norm block has a feed-forward with its norm and its gate, or none of them")
+        self.mixer, self.mixer_norm, self.mixer_gate = mixer, mixer_norm, mixer_gate
+        self.feed_forward, self.feed_forward_norm, self.feed_forward_gate = feed_forward, feed_forward_norm, feed_forward_gate
+
+    def forward(self, stream, ctx, cache):
+        h = self.mixer_norm.forward(stream)
+        logits = self.mixer_gate.logits(h)     # before the mixer: its input is the same rows
+        stream.delta = self.mixer.forward(h, ctx, cache)
+        stream.gate = (logits, self.mixer_gate.bias)
+        if self.feed_forward is not None:
+            h = self.feed_forward_norm.forward(stream)
+            logits = self.feed_forward_gate.logits(h)
+            stream.delta = self.feed_forward.forward(h, ctx)
+            stream.gate = (logits, self.feed_forward_gate.bias)

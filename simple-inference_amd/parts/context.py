@@ -74,14 +74,20 @@ class ResidualStream:
 
     ``lowered`` is the residual in the compute dtype, if the kernel that last changed the residual left it (a
     sublayer that reads the residual itself, not a norm of it, takes it from there); setting a delta forgets it.
+
+    ``gate`` belongs to the pending delta: ``(logits, bias)`` of an elementwise sigmoid gate that the delta passes
+    on its way into the residual (``residual += delta * sigmoid(logits + bias)``).  It is set after the delta and
+    forgotten with it; whoever adds the delta (a norm, ``settle``) reads it.  A delta may also be a
+    ``BiasedDelta``: a result whose bias is still to be added, which the gated add takes in passing.
     """
 
-    __slots__ = ("residual", "raw_delta", "lowered")
+    __slots__ = ("residual", "raw_delta", "lowered", "gate")
 
     def __init__(self, residual: torch.Tensor, delta: Optional[torch.Tensor] = None):
         self.residual = residual
         self.raw_delta = delta
         self.lowered = None
+        self.gate = None
 
     @property
     def delta(self):
@@ -92,5 +98,39 @@ class ResidualStream:
     @delta.setter
     def delta(self, value):
         self.raw_delta = value
+        self.gate = None
         if value is not None:
             self.lowered = None
+
+    def settle(self, kernels) -> torch.Tensor:
+        """Adds what is pending into the residual (no norm follows) and returns the residual."""
+        raw = self.raw_delta
+        if raw is None:
+            return self.residual
+        bias = None
+        if isinstance(raw, BiasedDelta):
+            raw, bias = raw.value(), raw.bias
+        elif hasattr(raw, "compute"):
+            raw = raw.compute()
+        gate, gate_bias = self.gate if self.gate is not None else (None, None)
+        kernels.gated_add(self.residual, raw, gate, gate_bias, bias)
+        self.delta = None
+        return self.residual
+
+
+class BiasedDelta:
+    """A sublayer's result whose bias is not added yet: ``y + bias``.  A sum that can take the bias in passing reads
+    ``value()`` and ``bias``; everybody else gets the tensor from ``compute()``."""
+
+    __slots__ = ("y", "bias", "kernels")
+
+    def __init__(self, y, bias, kernels):
+        self.y, self.bias, self.kernels = y, bias, kernels
+
+    def value(self):
+        if hasattr(self.y, "compute"):
+            self.y = self.y.compute()
+        return self.y
+
+    def compute(self):
+        return self.kernels.add_bias(self.value(), self.bias)

@@ -5,7 +5,8 @@ The embedding gathers rows of ``[V, H]`` into the float32 residual, multiplied b
 ``logits = h E^T``; tied, it uses the embedding's storage (reference:
 ``ops/embedding.py:78-86``); untied, it has a matrix of its own, which the
 reference mishandles by overwriting the embedding (``model/llama.py:147-154``).
-Logits leave the head as float32.
+Logits leave the head as float32; a head with a ``scale`` multiplies them by it, and one with a ``softcap`` ``c``
+then maps every logit ``z`` to ``c * tanh(z / c)``.
 """
 
 from __future__ import annotations
@@ -39,12 +40,16 @@ class TokenEmbedding:
 
 @register_head("head")
 class OutputHead:
-    """params: vocab_size, hidden_size, tied."""
+    """params: vocab_size, hidden_size, tied, and optionally scale and softcap."""
 
     def __init__(self, params, env):
         self.vocab = int(params["vocab_size"])
         self.hidden = int(params["hidden_size"])
         self.tied = bool(params["tied"])
+        self.scale = float(params.get("scale") or 1.0)
+        self.softcap = float(params["softcap"]) if params.get("softcap") else None
+        if self.softcap is not None and not self.softcap > 0:
+            raise ValueError(f"a soft cap must be positive, got {self.softcap}")
         self.env = env
         self.embedding = None
         self._weight = None
@@ -70,4 +75,7 @@ class OutputHead:
         return self.embedding.weight if self.tied else self._weight
 
     def forward(self, h):
-        return self.env.kernels.linear(h, self.weight, out_float32=True)
+        logits = self.env.kernels.linear(h, self.weight, out_float32=True)
+        if self.scale != 1.0 or self.softcap is not None:
+            logits = self.env.kernels.scale_softcap(logits, self.scale, self.softcap)
+        return logits

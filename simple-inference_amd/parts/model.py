@@ -15,7 +15,7 @@ import torch
 
 from .context import BuildEnv, LayerCache, ResidualStream, StepContext
 from .plan import ModelPlan, PagedKVNeed, StateNeed, TensorSpec
-from .registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS
+from .registry import BLOCKS, EMBEDDINGS, FEED_FORWARDS, GATES, HEADS, MIXERS, NORMS, STREAM_OPS
 
 
 @dataclass
@@ -35,7 +35,7 @@ class CacheLayout:
     run_state: List[Optional[int]] = field(default_factory=list)
 
 
-_REGISTRY_OF_ROLE = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS}
+_REGISTRY_OF_ROLE = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS, "gate": GATES}
 
 
 class _Layer:
@@ -68,7 +68,12 @@ class DecoderModel:
                 raise ValueError(f"the plan ties a {plan.head.kind!r} head to the embedding, but that head cannot share one")
             self.head.share_embedding(self.embedding)
         self.order = plan.run_order()
-        self._parts = [(self.embedding, plan.embedding)]
+        self.stream_ops = [STREAM_OPS.get(spec.kind)(spec.params, env) for spec in plan.stream_ops]
+        for e, i in plan.entries.items():
+            if not 0 <= e < len(self.order) or not 0 <= i < len(self.stream_ops):
+                raise ValueError(f"the plan enters run {e} through stream operation {i}: one of them does not exist")
+        self.entries = dict(plan.entries)
+        self._parts = [(self.embedding, plan.embedding)] + list(zip(self.stream_ops, plan.stream_ops))
         for layer in self.layers:
             self._parts.extend(layer.parts)
         self._parts += [(self.final_norm, plan.final_norm), (self.head, plan.head)]
@@ -135,8 +140,13 @@ class DecoderModel:
     # -- forward -----------------------------------------------------------
     def forward(self, ctx: StepContext, caches: List[LayerCache]) -> Optional[torch.Tensor]:
         """Runs the step's tokens; returns float32 logits ``[n_logit_rows, vocab]`` (None if none wanted)."""
-        stream = ResidualStream(self.embedding.forward(ctx))
+        first = self.embedding.forward(ctx)
+        # layers add into the residual in place: where a later stream operation wants the embedding output again,
+        # the stream starts from a second gather of it
+        stream = ResidualStream(self.embedding.forward(ctx) if self.entries and 0 not in self.entries else first)
         for e, li in enumerate(self.order):
+            if e in self.entries:
+                self.stream_ops[self.entries[e]].forward(stream, ctx, first)
             self.layers[li].block.forward(stream, ctx, caches[e])
         if ctx.n_logit_rows == 0:
             return None

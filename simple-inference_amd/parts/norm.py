@@ -10,6 +10,7 @@ the norm of what the sublayer returned, ``x += y * rsqrt(mean(y^2) + eps) * w``,
 
 from __future__ import annotations
 
+from .context import BiasedDelta
 from .plan import TensorSpec
 from .registry import register_norm
 
@@ -57,12 +58,33 @@ class RMSNorm:
         product's own kernel, and the product after the norm divides: the norm has no kernel of its own.
         """
         k = self.env.kernels
+        if stream.gate is not None or isinstance(stream.raw_delta, BiasedDelta):
+            return self._gated(stream, rows)
         if scaled_ok and rows is None and hasattr(stream.raw_delta, "compute") and hasattr(k, "linear_into_residual"):
             out = k.linear_into_residual(stream.raw_delta, stream.residual, self.weight, self.eps)
             stream.delta = None
             return out
         out = self.env.kernels.add_rmsnorm(
             stream.residual, stream.delta, self.weight, self.eps, self.env.dtype, rows)
+        if rows is None:
+            stream.delta = None
+        return out
+
+    def _gated(self, stream, rows):
+        """The same with a delta that passes an elementwise sigmoid gate (``stream.gate``) and may still lack its
+        bias: ``residual += (delta + bias) * sigmoid(gate logits + gate bias)``, all inside the norm's kernel."""
+        raw, bias = stream.raw_delta, None
+        if isinstance(raw, BiasedDelta):
+            raw, bias = raw.value(), raw.bias
+        elif hasattr(raw, "compute"):
+            raw = raw.compute()
+        logits, gate_bias = stream.gate if stream.gate is not None else (None, None)
+        if logits is None:      # a bias alone: nothing to fuse it into
+            raw, bias = self.env.kernels.add_bias(raw, bias), None
+            out = self.env.kernels.add_rmsnorm(stream.residual, raw, self.weight, self.eps, self.env.dtype, rows)
+        else:
+            out = self.env.kernels.add_rmsnorm(stream.residual, raw, self.weight, self.eps, self.env.dtype, rows,
+                                               gate=logits, gate_bias=gate_bias, delta_bias=bias)
         if rows is None:
             stream.delta = None
         return out

@@ -13,6 +13,9 @@ the part's own tensor names to the names in the checkpoint.
 * ``order`` lists layer indices in the order they run.  A layer may be named
   twice (each run keeps a cache of its own), and a mixer may read the cache
   that another layer's latest run wrote (``params["kv_from_layer"]``).
+* ``entries`` names, for some runs of the order, a stream operation that is applied to the residual stream right
+  before that run (a re-mix with the embedding output where a run of layers is walked again, for instance);
+  ``stream_ops`` holds their specs, so that several runs can share one operation and its tensors.
 """
 
 from __future__ import annotations
@@ -26,10 +29,10 @@ class PartSpec:
     kind: str
     params: Dict[str, Any] = field(default_factory=dict)
     weights: Dict[str, str] = field(default_factory=dict)
-    role: str = ""     # in a layer: which registry ``kind`` is looked up in ("mixer", "feed_forward", "norm")
+    role: str = ""     # in a layer: which registry ``kind`` is looked up in ("mixer", "feed_forward", "norm", "gate")
 
 
-ROLES = ("mixer", "feed_forward", "norm")
+ROLES = ("mixer", "feed_forward", "norm", "gate")
 
 
 @dataclass
@@ -89,6 +92,8 @@ class ModelPlan:
     max_position_embeddings: Optional[int] = None
     # checkpoint names that may be stored beside the parts' tensors -> the tensor each must then be equal to
     duplicates: Dict[str, str] = field(default_factory=dict)
+    stream_ops: List[PartSpec] = field(default_factory=list)
+    entries: Dict[int, int] = field(default_factory=dict)   # run of the order -> index into ``stream_ops``
 
     def run_order(self) -> List[int]:
         order = list(range(len(self.layers))) if self.order is None else list(self.order)
@@ -109,6 +114,9 @@ class TensorSpec:
     role "matrix": kept in the engine's compute dtype (bfloat16 or float32).
     role "vector": small gains and the like, held in float32 in both modes.
     role "table":  integers, held as int32.
+    role "float_matrix": a matrix whose products are taken in float32 in both modes (a router's).
+
+    A size of -1 is read from the checkpoint: the part learns it when its tensors are bound.
     """
 
     shape: Tuple[int, ...]

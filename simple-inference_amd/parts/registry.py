@@ -20,6 +20,10 @@ Interfaces (``env`` is a ``BuildEnv``; ``ctx`` a ``StepContext``):
 * block: ``__init__(self, **parts)`` with the names it gives its parts as keyword arguments (the pre-norm
   block: ``mixer, feed_forward, mixer_norm, feed_forward_norm``; a ``LayerSpec`` names the parts of its
   layer under those names), ``forward(stream, ctx, cache) -> None``.
+* gate (of a sublayer's result on its way into the residual stream): ``logits(h) -> Tensor[N, hidden]`` from
+  the sublayer's own input, and ``bias`` (float vector or None); the block hands both to the stream.
+* stream operation: ``forward(stream, ctx, first)`` changes the residual stream in place before a run of the order;
+  ``first`` is the embedding output of the step's tokens (float32).
 * embedding: ``forward(ctx) -> Tensor[N, hidden]`` float32, the residual stream's start.
 * head: ``forward(h) -> Tensor[rows, vocab]`` float32 logits; a head that can use the embedding's
   matrix has ``share_embedding(embedding)``, called before ``bind`` when its params say ``tied``.
@@ -65,6 +69,8 @@ POSITION_ENCODINGS = _Registry("position encoding")
 BLOCKS = _Registry("block")
 EMBEDDINGS = _Registry("embedding")
 HEADS = _Registry("head")
+GATES = _Registry("gate")
+STREAM_OPS = _Registry("stream operation")
 
 register_mixer: Callable = MIXERS.register
 register_feed_forward: Callable = FEED_FORWARDS.register
@@ -73,3 +79,5 @@ register_position_encoding: Callable = POSITION_ENCODINGS.register
 register_block: Callable = BLOCKS.register
 register_embedding: Callable = EMBEDDINGS.register
 register_head: Callable = HEADS.register
+register_gate: Callable = GATES.register
+register_stream_op: Callable = STREAM_OPS.register

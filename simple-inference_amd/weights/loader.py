@@ -10,7 +10,8 @@ that lists every missing tensor, every unexpected tensor and every wrong shape.
 Dtypes.  A tensor stored in bfloat16 (or float16) is kept in bfloat16 when the
 engine computes in bfloat16 and widened (exactly) when it computes in float32.
 A tensor stored in float32 stays float32 in both modes; integer tables become
-int32; small vectors (norm gains) are held in float32 whatever their storage.
+int32; small vectors (norm gains) are held in float32 whatever their storage, and so are
+matrices whose products are taken in float32 in both modes (a router's).
 """
 
 from __future__ import annotations
@@ -73,9 +74,14 @@ def _shard_map(folder: Path) -> Dict[str, Path]:
 def target_dtype(stored: torch.dtype, role: str, compute: torch.dtype) -> torch.dtype:
     if role == "table" or not stored.is_floating_point:
         return torch.int32
-    if role == "vector" or stored == torch.float32 or stored == torch.float64:
+    if role in ("vector", "float_matrix") or stored == torch.float32 or stored == torch.float64:
         return torch.float32
     return compute  # bfloat16 / float16 storage follows the engine
+
+
+def shape_fits(found, wanted) -> bool:
+    """Whether a stored shape is the wanted one; a wanted size of -1 takes any size (the part reads it from there)."""
+    return len(found) == len(wanted) and all(w == -1 or int(f) == int(w) for f, w in zip(found, wanted))
 
 
 def check_names_and_shapes(found: Mapping[str, Tuple[int, ...]], expected: Mapping[str, TensorSpec],
@@ -85,7 +91,7 @@ def check_names_and_shapes(found: Mapping[str, Tuple[int, ...]], expected: Mappi
     missing = [n for n in expected if n not in found]
     unexpected = [n for n in found if n not in expected and n not in duplicates and not (ignore and n.endswith(ignore))]
     wrong = [(n, tuple(found[n]), tuple(expected[n].shape)) for n in expected
-             if n in found and tuple(found[n]) != tuple(expected[n].shape)]
+             if n in found and not shape_fits(found[n], expected[n].shape)]
     wrong += [(n, tuple(found[n]), tuple(expected[other].shape)) for n, other in duplicates.items()
               if n in found and n not in expected and other in expected
               and tuple(found[n]) != tuple(expected[other].shape)]

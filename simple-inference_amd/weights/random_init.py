@@ -31,6 +31,9 @@ def random_tensors(expected: Mapping[str, TensorSpec], seed: int, std: float = 0
     for name, spec in expected.items():
         if spec.role == "table":
             raise ValueError(f"no random rule for integer table {name}")
+        if any(d < 0 for d in spec.shape):
+            raise ValueError(f"tensor {name} has a size that only a checkpoint gives ({spec.shape}): name it in the "
+                             f"configuration to draw random weights")
         t = torch.empty(spec.shape, dtype=torch.float32, device=device)
         if spec.role == "vector":
             t.normal_(0.0, 1.0, generator=gen).mul_(gain_std).add_(1.0)

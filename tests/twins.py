@@ -35,17 +35,104 @@ class TwinKernels:
         return residual if out_dtype == torch.float32 else residual.to(out_dtype)
 
     # -- residual add + rms norm ---------------------------------------------
-    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None):
+    def add_rmsnorm(self, residual, delta, weight, eps, out_dtype, rows=None, gate=None, gate_bias=None,
+                    delta_bias=None):
+        if delta is not None:
+            delta = self._gated(delta, gate, gate_bias, delta_bias)
         if rows is None:
             if delta is not None:
-                residual.add_(delta.float())
+                residual.add_(delta)
             x = residual
         else:
             x = residual[rows.long()]
             if delta is not None:
-                x = x + delta[rows.long()].float()
+                x = x + delta[rows.long()]
         var = x.pow(2).mean(-1, keepdim=True)
         return (x * torch.rsqrt(var + eps) * weight.float()).to(out_dtype)
+
+    @staticmethod
+    def _gated(delta, gate, gate_bias, delta_bias):
+        d = delta.float()
+        if delta_bias is not None:
+            d = d + delta_bias.float()
+        if gate is not None:
+            z = gate.float()
+            if gate_bias is not None:
+                z = z + gate_bias.float()
+            d = d * torch.sigmoid(z)
+        return d
+
+    def gated_add(self, residual, delta, gate=None, gate_bias=None, delta_bias=None):
+        residual.add_(self._gated(delta, gate, gate_bias, delta_bias))
+
+    def add_bias(self, y, bias):
+        y.copy_((y.float() + bias.float()).to(y.dtype))
+        return y
+
+    def head_gate(self, out, logits, n_heads):
+        n = out.shape[0]
+        gated = out.float().view(n, n_heads, -1) * torch.sigmoid(logits.float())[:, :, None]
+        out.copy_(gated.view(n, -1).to(out.dtype))
+        return out
+
+    def side_by_side(self, a, b, dtype):
+        return torch.cat([a, b], dim=-1).to(dtype)
+
+    def scale_softcap(self, logits, scale=1.0, cap=None):
+        logits.mul_(scale)
+        if cap is not None:
+            logits.copy_(cap * torch.tanh(logits / cap))
+        return logits
+
+    # -- linear attention with a state ------------------------------------------
+    def gla_recurrent(self, proj, columns, a2, a2_bias, norm_weight, n_heads, key_dim, value_dim, tau, q_scale, eps,
+                      ctx, cache):
+        N = proj.shape[0]
+        H, D, Dv, rank = n_heads, key_dim, value_dim, a2.shape[1]
+        cq, ck, cv, cg, ca = columns
+        p = proj.float()
+        q = p[:, cq:cq + H * D].view(N, H, D) * q_scale
+        k = p[:, ck:ck + H * D].view(N, H, D)
+        v = p[:, cv:cv + H * Dv].view(N, H, Dv)
+        g = p[:, cg:cg + H * Dv]
+        z = p[:, ca:ca + rank] @ a2.float().T
+        if a2_bias is not None:
+            z = z + a2_bias.float()
+        alpha = torch.exp(torch.nn.functional.logsigmoid(z) / tau).view(N, H, D)
+        out = torch.zeros(N, H, Dv)
+        cu, slots = ctx.cu_q.tolist(), ctx.state_slots.tolist()
+        for s in range(ctx.n_seqs):
+            S = cache.state[slots[s]]            # [H, D, Dv] float, updated in place
+            for t in range(cu[s], cu[s + 1]):
+                S.mul_(alpha[t][:, :, None]).add_(k[t][:, :, None] * v[t][:, None, :])
+                out[t] = torch.einsum("hd,hdv->hv", q[t], S)
+        out = out * torch.rsqrt(out.pow(2).mean(-1, keepdim=True) + eps) * norm_weight.float()
+        return (out.view(N, H * Dv) * torch.nn.functional.silu(g)).to(proj.dtype)
+
+    # -- mixture of experts ---------------------------------------------------------
+    def moe_route(self, h, router, top):
+        logits = h.float() @ router.float().T
+        order = torch.sort(logits, dim=-1, descending=True, stable=True).indices[:, :top]
+        best = torch.gather(logits, 1, order)
+        return order.to(torch.int32), torch.softmax(best, -1)
+
+    def moe_experts(self, h, w_gate_up, w_down, ids, weights, shared=None, shared_gate=None):
+        n, top = ids.shape
+        ff = w_gate_up.shape[1] // 2
+        x = h.float()
+        y = torch.zeros(n, w_down.shape[1])
+        for t in range(n):
+            for k in range(top):
+                e = int(ids[t, k])
+                gu = w_gate_up[e].float() @ x[t]
+                a = (torch.nn.functional.silu(gu[:ff]) * gu[ff:]).to(h.dtype).float()
+                y[t] += weights[t, k] * (w_down[e].float() @ a)
+        if shared is not None:
+            s = shared.float()
+            if shared_gate is not None:
+                s = s * torch.sigmoid(shared_gate.float())
+            y = y + s
+        return y.to(h.dtype)
 
     # -- matrix product ------------------------------------------------------
     def linear(self, x, w, out_float32=False):
@@ -74,20 +161,23 @@ class TwinKernels:
         return a.to(x.dtype)
 
     def qkv_to_cache(self, x, w_qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache,
-                     value_dim=None, bias=None, qk_norm=None):
+                     value_dim=None, bias=None, qk_norm=None, q_temp=None, extra_columns=0):
         qkv = self.linear(x, w_qkv)
         self.rope_kv_write(qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache,
-                           value_dim=value_dim, bias=bias, qk_norm=qk_norm)
+                           value_dim=value_dim, bias=bias, qk_norm=qk_norm, q_temp=q_temp)
+        if extra_columns:
+            return qkv, qkv[:, qkv.shape[1] - extra_columns:]
         return qkv
 
     # -- rotation + cache write ----------------------------------------------
     def rope_kv_write(self, qkv, n_heads, n_kv_written, head_dim, rotary_dim, cos, sin, ctx, cache,
-                      value_dim=None, bias=None, qk_norm=None):
+                      value_dim=None, bias=None, qk_norm=None, q_temp=None):
         N = qkv.shape[0]
         pos = ctx.positions.long()
         value_dim = value_dim or head_dim
         if bias is not None:
-            qkv.copy_((qkv.float() + bias.float()).to(qkv.dtype))
+            own = bias.numel()
+            qkv[:, :own] = (qkv[:, :own].float() + bias.float()).to(qkv.dtype)
         q = qkv[:, :n_heads * head_dim].view(N, n_heads, head_dim)
 
         def normed(x, gain):
@@ -109,7 +199,11 @@ class TwinKernels:
             out[..., half:rotary_dim] = b * c + a * s
             return out.to(x.dtype)
 
-        q.copy_(rotate(normed(q, qk_norm[0] if qk_norm else None)))
+        qn = normed(q, qk_norm[0] if qk_norm else None)
+        if q_temp is not None:
+            temp = 1.0 + q_temp[0] * torch.log((torch.div(pos + 1, q_temp[1], rounding_mode="floor") + 1).float())
+            qn = (qn.float() * temp[:, None, None]).to(q.dtype)
+        q.copy_(rotate(qn))
         if n_kv_written == 0:
             return
         kv0 = n_heads * head_dim
