@@ -24,6 +24,8 @@ prefix reuse.  They print one JSON line of their own kind.
 1B, 3B and 8B widths, head counts and feed-forward sizes; ``--layers`` layers of each, default 8; seeded random
 weights): decode at batch 8 and 1 over 2,048-token contexts and the prefill of 2,048 tokens, each with its
 fraction of the HBM or matrix-core roofline, in one JSON line of its own kind.
+``--workload mogisun`` does the same for the Mogisun design: a model of softmax-attention layers with dense
+feed-forwards and a model of linear-attention layers with routed experts, each beside the Llama model.
 
 The engine runs on one GPU; asked for more it says so and exits with 2.
 """
@@ -76,9 +78,10 @@ def parse_args(argv=None):
     ap.add_argument("--temperature", type=float, default=0.0, help="sampling of the decode measurement (0: greedy)")
     ap.add_argument("--top-k", type=int, default=0)
     ap.add_argument("--top-p", type=float, default=1.0)
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "shared-prefix", "feduzen"])
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "shared-prefix", "feduzen", "mogisun"])
     ap.add_argument("--shapes", default="1b,3b,8b", help="--workload feduzen: which layer sizes, comma separated")
-    ap.add_argument("--models", default="feduzen,llama", help="--workload feduzen: which of the two models to run")
+    ap.add_argument("--models", default=None, help="--workload feduzen or mogisun: which of the models to run "
+                    "(feduzen,llama; mogisun-attention,mogisun-linear,llama)")
     ap.add_argument("--max-running", type=int, default=64, help="request slots of the stream workloads")
     return ap.parse_args(argv)
 
@@ -368,7 +371,7 @@ def feduzen_workload(args):
         kv_bytes = 2 * layers * kv * el
         for model, cfg, ff_w, head_w in (("feduzen", feduzen_config_like(llama, layers), 2 * H * I, V * H),
                                          ("llama", llama, 3 * H * I, V * H)):
-            if model not in args.models.split(","):
+            if model not in (args.models or "feduzen,llama").split(","):
                 continue
             ecfg = EngineConfig(max_running=8, max_seq_len=max(4096, -(-total_len // 1024) * 1024), dtype=args.dtype,
                                 chunk_tokens=max(2048, T), eos_id=-1, use_graphs=not args.no_graphs, device="cuda:0")
@@ -395,6 +398,71 @@ def feduzen_workload(args):
             "config": {"layers": layers, "context": context, "prefill_tokens": T, "shapes": FEDUZEN_SHAPES,
                        "feduzen": "full rotation, q/k norm, biases, sinks, a block mask wider than the context, "
                                   "dense relu^2 feed-forward (two matrices where the gated one has three)"},
+            "shapes": out}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+def mogisun_config_like(llama_cfg, layers, kind):
+    """A Mogisun config.json with the widths, head counts and feed-forward size of a Llama one.  ``attention``: every
+    layer softmax attention and a dense feed-forward (the Llama layer plus the design's gates, norms and
+    temperature).  ``linear``: every layer gated linear attention with as many heads of the same width, and eight
+    experts of a quarter of the feed-forward size, two a token, beside a shared expert of half of it (as many active
+    feed-forward weights as the dense layer has).  All layers are one walk of a loop, so the re-mix runs once."""
+    dim, heads = llama_cfg["head_dim"], llama_cfg["num_attention_heads"]
+    ff = llama_cfg["intermediate_size"]
+    if kind == "attention":
+        layer = {"type": "attention", "mlp": {"kind": "dense", "ff": ff},
+                 "mixer": {"dim": dim, "vdim": dim, "heads": heads, "kv_heads": llama_cfg["num_key_value_heads"],
+                           "scale": dim ** -0.5, "q_temp": {"coef": 0.1, "every": 1024}}}
+    else:
+        layer = {"type": "gla", "mixer": {"dim": dim, "vdim": dim, "heads": heads, "tau": 16.0, "rank": 64},
+                 "mlp": {"kind": "moe", "router": {"experts": 8, "top": 2}, "expert": {"ff": ff // 4},
+                         "shared": {"ff": ff // 2}}}
+    return {"architecture": "Mogisun", "vocab": llama_cfg["vocab_size"], "width": llama_cfg["hidden_size"],
+            "norm": {"eps": llama_cfg["rms_norm_eps"]}, "logit_scale": 1.0, "logit_softcap": 30.0,
+            "loop": {"start": 0, "stop": layers, "times": 1},
+            "layers": [json.loads(json.dumps(layer)) for _ in range(layers)]}
+
+
+def mogisun_workload(args):
+    """Decode and prefill of the Mogisun design (its two kinds of layer, each alone) beside the Llama model at equal
+    layer sizes."""
+    from simple_inference_amd import Engine, EngineConfig, preset
+
+    layers = args.layers or 8
+    dt_name = "bf16" if args.dtype == "bfloat16" else "fp32"
+    context, T = args.context, args.prefill_tokens
+    total_len = max(context + args.warmup + args.steps + decode_allowance(max(2048, T), 8, context), T + 2)
+    wanted = (args.models or "mogisun-attention,mogisun-linear,llama").split(",")
+    out = {}
+    for shape in [x for x in args.shapes.split(",") if x]:
+        llama = preset(FEDUZEN_SHAPES[shape])
+        llama["num_hidden_layers"] = layers
+        for model, cfg in (("mogisun-attention", mogisun_config_like(llama, layers, "attention")),
+                           ("mogisun-linear", mogisun_config_like(llama, layers, "linear")), ("llama", llama)):
+            if model not in wanted:
+                continue
+            ecfg = EngineConfig(max_running=8, max_seq_len=max(4096, -(-total_len // 1024) * 1024), dtype=args.dtype,
+                                chunk_tokens=max(2048, T), eos_id=-1, use_graphs=not args.no_graphs, device="cuda:0")
+            ecfg.num_kv_blocks = 8 * (-(-total_len // ecfg.block_size)) + 8
+            engine = Engine.from_random(cfg, seed=args.seed, engine_cfg=ecfg, std=0.02, generate_on_device=True)
+            row = {}
+            for batch in (8, 1):
+                dt, _ = measure_decode(engine, batch, context, args.steps, args.warmup, args.seed)
+                row[f"decode_b{batch}"] = {"tok_s": round(batch / dt, 1), "ms_per_step": round(dt * 1e3, 4)}
+            if not args.no_prefill:
+                sec, best = measure_prefill(engine, T)
+                row["prefill"] = {"tok_s": round(T / sec, 1), "ms": round(sec * 1e3, 3), "best_ms": round(best * 1e3, 3)}
+            out.setdefault(shape, {})[model] = row
+            del engine
+            torch.cuda.empty_cache()
+    line = {"metric": "Mogisun beside Llama at equal layer sizes: decode tok/s (batch 8, 1) and prefill tok/s",
+            "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "dtype": dt_name,
+            "data": "synthetic (seeded random weights and uniform-random token ids)",
+            "config": {"layers": layers, "context": context, "prefill_tokens": T, "shapes": FEDUZEN_SHAPES,
+                       "mogisun-attention": "softmax attention with its gates, norms and temperature, dense SwiGLU",
+                       "mogisun-linear": "gated linear attention, 8 experts of ff/4 (2 a token) and a shared one of ff/2"},
             "shapes": out}
     print(json.dumps(line), flush=True)
     return 0
@@ -468,6 +536,8 @@ def main(argv=None):
         return 1
     if args.workload == "feduzen":
         return feduzen_workload(args)
+    if args.workload == "mogisun":
+        return mogisun_workload(args)
     if args.workload != "decode":
         return stream_workload(args)
     points = [int(p) for p in args.points.split(",") if p]

@@ -45,6 +45,7 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
             const int ow = __shfl_xor(which, off, SIA_WAVE);
             if (ob > best || (ob == best && ow < which)) { best = ob; which = ow; }
         }
+        if (which >= n_experts) which = k;   // logits that are not numbers order nothing: still an expert that exists
         if (k == 0) first = best;
         const float p = expf(best - first);
         total += p;
@@ -177,5 +178,190 @@ SIA_EXPORT int sia_moe_down(const void* act, const void* w2, const int* ids, con
                            width, ff, top, vec);
     else
         return SIA_BAD_ARGUMENT;
+    return SIA_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Steps of many tokens (bfloat16): the slots are sorted by expert on the device and the experts' products run on the
+// matrix cores, a tile of 32 slots of one expert at a time.
+//
+//   sort:     counts the slots of every expert, gives every expert whole tiles of 32 places (the places a tile does
+//             not fill hold -1) and writes, for every place, its slot, and for every tile, its expert.  One workgroup;
+//             nothing comes back to the host: the products are launched for the most tiles there can be
+//             (ceil(slots / 32) + experts) and the tiles beyond the count leave at once.  Which place of its expert's
+//             tiles a slot gets depends on the order of atomic adds; a slot's numbers do not (a row of a product
+//             does not depend on the other rows).
+//   gate/up:  a[s, f] for a tile's slots and 128 columns f a workgroup: v_mfma_f32_16x16x32_bf16 with the weights'
+//             rows as the first operand and the tokens' rows as the second, both read from memory k-contiguous
+//             (lane (r, g): row r, elements 8g .. 8g + 7 of a step of 32); a wave holds 32 columns x 32 slots of
+//             gate and of up and writes 4 consecutive columns of a slot at a time.
+//   down:     y[s, c] the same way, bfloat16, one row per slot;
+//   combine:  out[n, c] = sum_k weights[n, k] * y[n * top + k, c] (+ sigmoid(sg[n]) * shared[n, c]), float sums.
+// ---------------------------------------------------------------------------------------------------------------
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 moe_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float moe_floatx4;
+
+#define MOE_TILE 32
+
+__global__ __launch_bounds__(1024) void moe_sort_kernel(const int* __restrict__ ids, int n_slots, int n_experts,
+                                                        int* __restrict__ place_slot, int* __restrict__ tile_expert,
+                                                        int* __restrict__ n_tiles_out, int max_tiles) {
+    __shared__ int count_s[MOE_MAX_EXPERTS];
+    __shared__ int first_s[MOE_MAX_EXPERTS];   // first place of the expert's tiles
+    for (int e = threadIdx.x; e < n_experts; e += blockDim.x) count_s[e] = 0;
+    for (int i = threadIdx.x; i < max_tiles * MOE_TILE; i += blockDim.x) place_slot[i] = -1;
+    __syncthreads();
+    auto expert_of = [&](int s) { return min(max(ids[s], 0), n_experts - 1); };
+    for (int s = threadIdx.x; s < n_slots; s += blockDim.x) atomicAdd(&count_s[expert_of(s)], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int tile = 0;
+        for (int e = 0; e < n_experts; ++e) {
+            first_s[e] = tile * MOE_TILE;
+            const int tiles = (count_s[e] + MOE_TILE - 1) / MOE_TILE;
+            for (int t = 0; t < tiles; ++t) tile_expert[tile + t] = e;
+            tile += tiles;
+            count_s[e] = 0;   // from here on: the next free place of the expert
+        }
+        *n_tiles_out = tile;
+    }
+    __syncthreads();
+    for (int s = threadIdx.x; s < n_slots; s += blockDim.x) {
+        const int e = expert_of(s);
+        place_slot[first_s[e] + atomicAdd(&count_s[e], 1)] = s;
+    }
+}
+
+__device__ __forceinline__ moe_bf16x8 moe_ld8(const bf16_t* p) { return *reinterpret_cast<const moe_bf16x8*>(p); }
+
+// GATED: rows f and ff + f of W make silu(gate) * up; else a plain product.  Output row stride n_out.
+template <bool GATED>
+__global__ __launch_bounds__(256) void moe_tile_kernel(const bf16_t* __restrict__ x, int rows_per_slot,
+                                                       const bf16_t* __restrict__ w, const int* __restrict__ place_slot,
+                                                       const int* __restrict__ tile_expert,
+                                                       const int* __restrict__ n_tiles, bf16_t* __restrict__ out,
+                                                       int K, int n_out) {
+    const int tile = blockIdx.x;
+    if (tile >= *n_tiles) return;
+    const int wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE, r = lane & 15, g = lane >> 4;
+    const int e = tile_expert[tile];
+    const int c0 = blockIdx.y * 128 + wave * 32;          // this wave's 32 output columns
+    if (c0 >= n_out) return;
+    const size_t expert_rows = GATED ? 2 * (size_t)n_out : (size_t)n_out;
+    const bf16_t* we = w + (size_t)e * expert_rows * K;
+    int slot[2];
+    const bf16_t* xp[2];
+    const bf16_t* wp[2][2];
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) {
+        slot[mb] = place_slot[tile * MOE_TILE + mb * 16 + r];
+        xp[mb] = x + (size_t)(max(slot[mb], 0) / rows_per_slot) * K + g * 8;
+    }
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb) {
+        const int c = min(c0 + nb * 16 + r, n_out - 1);
+        wp[nb][0] = we + (size_t)c * K + g * 8;
+        wp[nb][1] = we + (size_t)(n_out + c) * K + g * 8;     // the up rows (GATED only)
+    }
+    moe_floatx4 acc[2][2][2];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) acc[nb][mb][h] = moe_floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < K; k += 32) {
+        moe_bf16x8 a[2][2], b[2];
+#pragma unroll
+        for (int mb = 0; mb < 2; ++mb) b[mb] = moe_ld8(xp[mb] + k);
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            a[nb][0] = moe_ld8(wp[nb][0] + k);
+            if (GATED) a[nb][1] = moe_ld8(wp[nb][1] + k);
+        }
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+            for (int mb = 0; mb < 2; ++mb) {
+                acc[nb][mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nb][0], b[mb], acc[nb][mb][0], 0, 0, 0);
+                if (GATED)
+                    acc[nb][mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[nb][1], b[mb], acc[nb][mb][1], 0, 0, 0);
+            }
+    }
+    // acc[nb][mb][.][i]: column c0 + nb * 16 + 4g + i of the slot at place mb * 16 + r
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb) {
+        if (slot[mb] < 0) continue;
+        const size_t row = GATED ? (size_t)slot[mb] : (size_t)slot[mb];
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            const int c = c0 + nb * 16 + 4 * g;
+            bf16_t v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float y = acc[nb][mb][0][i];
+                if (GATED) y = y / (1.f + expf(-y)) * acc[nb][mb][1][i];
+                v[i] = float_to_bf16(y);
+            }
+            bf16_t* dst = out + row * n_out + c;
+            if (c + 3 < n_out && n_out % 4 == 0) {
+                *reinterpret_cast<uint2*>(dst) = make_uint2((uint32_t)v[0] | ((uint32_t)v[1] << 16),
+                                                            (uint32_t)v[2] | ((uint32_t)v[3] << 16));
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (c + i < n_out) dst[i] = v[i];
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void moe_combine_kernel(const bf16_t* __restrict__ y, const float* __restrict__ weights,
+                                                          const bf16_t* __restrict__ shared,
+                                                          const bf16_t* __restrict__ shared_gate, int shared_gate_stride,
+                                                          bf16_t* __restrict__ out, int width, int top) {
+    const int n = blockIdx.x;
+    float scale = 1.f;
+    if (shared && shared_gate) scale = 1.f / (1.f + expf(-bf16_to_float(shared_gate[(size_t)n * shared_gate_stride])));
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        float acc = 0.f;
+        for (int k = 0; k < top; ++k)
+            acc += weights[(size_t)n * top + k] * bf16_to_float(y[((size_t)n * top + k) * width + c]);
+        if (shared) acc += scale * bf16_to_float(shared[(size_t)n * width + c]);
+        out[(size_t)n * width + c] = float_to_bf16(acc);
+    }
+}
+
+// ints of workspace the tiled form needs for a step of n_tokens (0: the step is too small for it, or the sizes
+// do not fit: the slot-by-slot form runs)
+SIA_EXPORT long long sia_moe_tiled_workspace(int n_tokens, int top, int n_experts, int width, int ff) {
+    const long long slots = (long long)n_tokens * top;
+    if (slots < 64 || width % 32 || ff % 32 || slots > 0x3fffffffLL) return 0;
+    const long long max_tiles = (slots + MOE_TILE - 1) / MOE_TILE + n_experts;
+    return max_tiles * MOE_TILE + max_tiles + 4;
+}
+
+// act [slots, ff] and y [slots, width] are the caller's scratch (bfloat16).
+SIA_EXPORT int sia_moe_tiled(const void* h, const void* w1, const void* w2, const int* ids, const float* weights,
+                             const void* shared, const void* shared_gate, int shared_gate_stride, void* act, void* y,
+                             void* out, int* workspace, int n_tokens, int width, int ff, int top, int n_experts,
+                             hipStream_t stream) {
+    if (n_tokens <= 0) return 0;
+    if (sia_moe_tiled_workspace(n_tokens, top, n_experts, width, ff) == 0 || n_experts > MOE_MAX_EXPERTS ||
+        (shared_gate && !shared))
+        return SIA_BAD_ARGUMENT;
+    const int slots = n_tokens * top;
+    const int max_tiles = (slots + MOE_TILE - 1) / MOE_TILE + n_experts;
+    int* place_slot = workspace;
+    int* tile_expert = workspace + (size_t)max_tiles * MOE_TILE;
+    int* n_tiles = tile_expert + max_tiles;
+    hipLaunchKernelGGL(moe_sort_kernel, dim3(1), dim3(1024), 0, stream, ids, slots, n_experts, place_slot, tile_expert,
+                       n_tiles, max_tiles);
+    hipLaunchKernelGGL(moe_tile_kernel<true>, dim3(max_tiles, (ff + 127) / 128), dim3(256), 0, stream,
+                       (const bf16_t*)h, top, (const bf16_t*)w1, place_slot, tile_expert, n_tiles, (bf16_t*)act, width, ff);
+    hipLaunchKernelGGL(moe_tile_kernel<false>, dim3(max_tiles, (width + 127) / 128), dim3(256), 0, stream,
+                       (const bf16_t*)act, 1, (const bf16_t*)w2, place_slot, tile_expert, n_tiles, (bf16_t*)y, ff, width);
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(256), 0, stream, (const bf16_t*)y, weights,
+                       (const bf16_t*)shared, (const bf16_t*)shared_gate, shared_gate_stride, (bf16_t*)out, width, top);
     return SIA_LAUNCH_CHECK();
 }

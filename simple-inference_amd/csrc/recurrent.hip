@@ -12,23 +12,31 @@
 // offsets); y is written as [tokens, H * Dv].  Products' results come in the compute type; decays, their logarithms,
 // the state, the sums over channels, the norm and the gate are float, with one rounding of y.
 //
+// The decays of all tokens and channels are computed first, by a kernel of their own (they do not depend on the
+// state, and a step's tokens are thousands of independent little products), into a float workspace.
 // A workgroup owns one (sequence, head) and walks the sequence's tokens of this step in order, so a request's
 // numbers depend on its own tokens only: not on how its prompt was cut, nor on what else the step holds.
 // Thread (j, r) keeps rows r, r + R, r + 2R, ... of column j of S in registers (R a power of two: the lanes of a
 // column are neighbours and add their shares of o by lane exchanges).  Blocks of a few tokens are staged through
 // LDS (q, k, alpha, v, g as floats), walked, and their outputs normed and gated a token a wave.
+//
+// A step with few (sequence, head) pairs and runs of many tokens (a prompt) would leave most of the chip idle, and
+// the walk along a sequence cannot be shortened.  Such a step gives every pair several workgroups, each with a
+// slice of the state's columns (they are independent of one another), more lanes per column and fewer rows per
+// lane; the outputs go to a float workspace and a second kernel norms and gates them, since a norm spans a head.
 #include "common.h"
 
 __device__ __forceinline__ float log_sigmoid(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
 template <typename T, int ROWS>
 __global__ __launch_bounds__(512) void gla_recurrent_kernel(
-    const T* __restrict__ proj, int row_stride, int q_col, int k_col, int v_col, int g_col, int a_col,
-    const T* __restrict__ a2, const float* __restrict__ a2_bias, const float* __restrict__ norm_w,
-    float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ slots, T* __restrict__ out,
-    int n_heads, int D, int Dv, int rank, int R, int block_tokens, float tau_inv, float q_scale, float eps) {
+    const T* __restrict__ proj, int row_stride, int q_col, int k_col, int v_col, int g_col,
+    const float* __restrict__ alpha, const float* __restrict__ norm_w, float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ slots, T* __restrict__ out,
+    int n_heads, int D, int Dv, int R, int block_tokens, float q_scale, float eps, int slice,
+    float* __restrict__ raw_out) {
     extern __shared__ float lds[];
     const int seq = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
+    const int j0 = blockIdx.z * slice;     // this workgroup's columns: j0 .. j0 + slice - 1
     const int first = cu_q[seq], last = cu_q[seq + 1];
     if (first >= last) return;
     const int TB = block_tokens;
@@ -38,10 +46,9 @@ __global__ __launch_bounds__(512) void gla_recurrent_kernel(
     float* v_s = al_s + TB * D;        // [TB][Dv]
     float* g_s = v_s + TB * Dv;        // [TB][Dv]
     float* o_s = g_s + TB * Dv;        // [TB][Dv]
-    float* a_s = o_s + TB * Dv;        // [TB][rank]
 
-    const int j = tid / R, r = tid % R;
-    const bool owns = j < Dv;
+    const int j = j0 + tid / R, r = tid % R;
+    const bool owns = tid / R < slice && j < Dv;
     float* S_mem = state + ((size_t)slots[seq] * n_heads + head) * D * Dv;
     float S[ROWS];
 #pragma unroll
@@ -53,26 +60,18 @@ __global__ __launch_bounds__(512) void gla_recurrent_kernel(
 
     for (int t0 = first; t0 < last; t0 += TB) {
         const int nt = min(TB, last - t0);
-        for (int idx = tid; idx < nt * rank; idx += blockDim.x) {
-            const int t = idx / rank, c = idx % rank;
-            a_s[idx] = to_float(proj[(size_t)(t0 + t) * row_stride + a_col + c]);
-        }
         for (int idx = tid; idx < nt * Dv; idx += blockDim.x) {
             const int t = idx / Dv, c = idx % Dv;
             const T* row = proj + (size_t)(t0 + t) * row_stride;
             v_s[t * Dv + c] = to_float(row[v_col + head * Dv + c]);
             g_s[t * Dv + c] = to_float(row[g_col + head * Dv + c]);
         }
-        __syncthreads();
         for (int idx = tid; idx < nt * D; idx += blockDim.x) {
             const int t = idx / D, c = idx % D;
             const T* row = proj + (size_t)(t0 + t) * row_stride;
             q_s[t * D + c] = to_float(row[q_col + head * D + c]) * q_scale;
             k_s[t * D + c] = to_float(row[k_col + head * D + c]);
-            const T* w = a2 + (size_t)(head * D + c) * rank;
-            float z = a2_bias ? a2_bias[head * D + c] : 0.f;
-            for (int m = 0; m < rank; ++m) z += a_s[t * rank + m] * to_float(w[m]);
-            al_s[t * D + c] = expf(log_sigmoid(z) * tau_inv);
+            al_s[t * D + c] = alpha[((size_t)(t0 + t) * n_heads + head) * D + c];
         }
         __syncthreads();
         for (int t = 0; t < nt; ++t) {
@@ -87,9 +86,13 @@ __global__ __launch_bounds__(512) void gla_recurrent_kernel(
                 }
             }
             for (int o = R / 2; o > 0; o >>= 1) acc += __shfl_xor(acc, o, SIA_WAVE);
-            if (owns && r == 0) o_s[t * Dv + j] = acc;
+            if (owns && r == 0) {
+                if (raw_out) raw_out[((size_t)(t0 + t) * n_heads + head) * Dv + j] = acc;
+                else o_s[t * Dv + j] = acc;
+            }
         }
         __syncthreads();
+        if (raw_out) continue;   // uniform: the norm is another kernel's
         for (int t = wave; t < nt; t += n_waves) {
             float ss = 0.f;
             for (int c = lane; c < Dv; c += SIA_WAVE) ss += o_s[t * Dv + c] * o_s[t * Dv + c];
@@ -109,32 +112,319 @@ __global__ __launch_bounds__(512) void gla_recurrent_kernel(
     }
 }
 
+// Sum over the 16 lanes of a row of a wave by lane exchanges inside the vector unit (no trip through LDS's crossbar):
+// neighbours, pairs of a quad, the mirrored half, the mirrored row.  Every lane of the row gets the sum.
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));    // quad_perm [1,0,3,2]
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));    // quad_perm [2,3,0,1]
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));   // row_half_mirror
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));   // row_mirror
+    return v;
+}
+
+// The walk alone, for a prompt's step in bfloat16 whose heads' columns are shared out (D a multiple of 8, rows and
+// columns aligned to 16 bytes).  The 16 lanes of one row of a wave share two or four columns of the state, lane r
+// keeping rows r * ROWS .. r * ROWS + ROWS - 1 of each (what a lane reads of q, k and the decays serves all its
+// columns: LDS bandwidth, which every lane's reads of the same numbers would exhaust, is spent once per
+// those columns); a token's outputs are sums over the row.  q, k and the decays lie in LDS so that the 16
+// lanes' 16-byte pieces of a read are one contiguous run (no bank meets twice).  Blocks of 32 tokens: their q, k
+// (16-byte pieces), decays (float4) and values are requested into registers while the block before is walked, so
+// that the walk never waits for memory.  Outputs go to the float workspace; the norm is the finishing kernel's.
+#define GLA_WALK_TOKENS 32
+#define GLA_WALK_THREADS 256
+template <int ROWS, int GLA_WALK_COLS>
+__global__ __launch_bounds__(GLA_WALK_THREADS) void gla_walk_kernel(
+    const bf16_t* __restrict__ proj, int row_stride, int q_col, int k_col, int v_col, const float* __restrict__ alpha,
+    float* __restrict__ state, const int* __restrict__ cu_q, const int* __restrict__ slots, int n_heads, int D, int Dv,
+    float q_scale, float* __restrict__ raw_out) {
+    extern __shared__ float lds[];
+    constexpr int TB = GLA_WALK_TOKENS, C = GLA_WALK_COLS, threads = GLA_WALK_THREADS;
+    constexpr int slice = threads / 16 * C;      // columns a workgroup
+    constexpr int Dp = 16 * ROWS;                // D filled up to the rows the lanes hold: what lies beyond D is zero
+    const int seq = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
+    const int j0 = blockIdx.z * slice;
+    const int first = cu_q[seq], last = cu_q[seq + 1];
+    if (first >= last) return;
+    float* q_s = lds;               // [TB][Dp], row d = r * ROWS + i at (i / 4) * 64 + r * 4 + i % 4
+    float* k_s = q_s + TB * Dp;
+    float* al_s = k_s + TB * Dp;
+    float* v_s = al_s + TB * Dp;    // [TB][slice]
+    float* o_s = v_s + TB * slice;  // [TB][slice]: a block's outputs, written out together
+    auto place = [](int d) { const int r = d / ROWS, i = d % ROWS; return (i / 4) * 64 + r * 4 + i % 4; };
+    for (int i = tid; i < 3 * TB * Dp; i += threads) lds[i] = 0.f;
+    const int jl = (tid / 16) * C, r = tid % 16;      // this lane's first column inside the slice, and its rows
+    float* S_mem = state + ((size_t)slots[seq] * n_heads + head) * D * Dv;
+    float S[C][ROWS];
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) {
+            const int d = r * ROWS + i, j = j0 + jl + c;
+            S[c][i] = (j < Dv && d < D) ? S_mem[(size_t)d * Dv + j] : 0.f;
+        }
+    const int d8 = D / 8, d4 = D / 4;
+    uint4 rq[4], rk[4];
+    float4 ra[8];
+    float rv[TB * slice / threads];     // a block's values: 32 tokens x 16 C columns over 256 threads
+    auto request = [&](int t0) {   // the block's pieces into registers; pieces beyond the sequence's end are not read
+        const int nt = min(TB, last - t0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int idx = tid + i * threads;
+            if (idx < nt * d8) {
+                const bf16_t* row = proj + (size_t)(t0 + idx / d8) * row_stride + head * D + (idx % d8) * 8;
+                rq[i] = *reinterpret_cast<const uint4*>(row + q_col);
+                rk[i] = *reinterpret_cast<const uint4*>(row + k_col);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int idx = tid + i * threads;
+            if (idx < nt * d4)
+                ra[i] = *reinterpret_cast<const float4*>(alpha + ((size_t)(t0 + idx / d4) * n_heads + head) * D + (idx % d4) * 4);
+        }
+#pragma unroll
+        for (int i = 0; i < TB * slice / threads; ++i) {
+            const int idx = tid + i * threads;
+            if (idx < nt * slice && j0 + idx % slice < Dv)
+                rv[i] = bf16_to_float(proj[(size_t)(t0 + idx / slice) * row_stride + v_col + head * Dv + j0 + idx % slice]);
+        }
+    };
+    auto deposit = [&](int t0) {
+        const int nt = min(TB, last - t0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int idx = tid + i * threads;
+            if (idx < nt * d8) {
+                const int base = (idx / d8) * Dp, d0 = (idx % d8) * 8;
+                // two 16-bit halves of a word are rows d and d + 1; no arrays, so that all of it stays in registers
+#define GLA_PUT(word_q, word_k, d)                                                                \
+    do {                                                                                          \
+        const int p0 = base + place(d), p1 = base + place((d) + 1);                               \
+        q_s[p0] = __uint_as_float((word_q) << 16) * q_scale;                                      \
+        q_s[p1] = __uint_as_float((word_q) & 0xffff0000u) * q_scale;                              \
+        k_s[p0] = __uint_as_float((word_k) << 16);                                                \
+        k_s[p1] = __uint_as_float((word_k) & 0xffff0000u);                                        \
+    } while (0)
+                GLA_PUT(rq[i].x, rk[i].x, d0);
+                GLA_PUT(rq[i].y, rk[i].y, d0 + 2);
+                GLA_PUT(rq[i].z, rk[i].z, d0 + 4);
+                GLA_PUT(rq[i].w, rk[i].w, d0 + 6);
+#undef GLA_PUT
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int idx = tid + i * threads;
+            if (idx < nt * d4) {
+                const int base = (idx / d4) * Dp, d0 = (idx % d4) * 4;   // four rows of one lane (ROWS is a multiple of 4)
+                *reinterpret_cast<float4*>(al_s + base + place(d0)) = ra[i];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < TB * slice / threads; ++i) {
+            const int idx = tid + i * threads;
+            if (idx < nt * slice) v_s[idx] = (j0 + idx % slice < Dv) ? rv[i] : 0.f;
+        }
+    };
+    // One round before the first block only requests it (each of the two steps is written once, so that the pieces
+    // on their way stay in registers).
+    for (int t0 = first - TB; t0 < last; t0 += TB) {
+        const int nt = min(TB, last - t0);
+        if (t0 >= first) deposit(t0);
+        __syncthreads();   // in the first round: the zeros are in place before the first pieces land on them
+        if (t0 + TB < last) request(t0 + TB);
+        if (t0 < first) continue;   // uniform
+        // a token's q, k and decays are read from LDS while the token before is worked on
+        float4 qn[ROWS / 4], kn[ROWS / 4], an[ROWS / 4];
+        auto fetch = [&](int t) {
+#pragma unroll
+            for (int i = 0; i < ROWS / 4; ++i) {
+                const int at = t * Dp + i * 64 + r * 4;
+                qn[i] = *reinterpret_cast<const float4*>(q_s + at);
+                kn[i] = *reinterpret_cast<const float4*>(k_s + at);
+                an[i] = *reinterpret_cast<const float4*>(al_s + at);
+            }
+        };
+        fetch(0);
+        for (int t = 0; t < nt; ++t) {
+            float4 qv[ROWS / 4], kv[ROWS / 4], av[ROWS / 4];
+            float vv[C];
+#pragma unroll
+            for (int i = 0; i < ROWS / 4; ++i) { qv[i] = qn[i]; kv[i] = kn[i]; av[i] = an[i]; }
+#pragma unroll
+            for (int c = 0; c < C; ++c) vv[c] = v_s[t * slice + jl + c];
+            fetch(min(t + 1, TB - 1));
+#pragma unroll
+            for (int c = 0; c < C; ++c) {
+                const float v = vv[c];
+                float acc = 0.f;
+#pragma unroll
+                for (int i = 0; i < ROWS / 4; ++i) {
+                    S[c][4 * i] = av[i].x * S[c][4 * i] + kv[i].x * v;
+                    S[c][4 * i + 1] = av[i].y * S[c][4 * i + 1] + kv[i].y * v;
+                    S[c][4 * i + 2] = av[i].z * S[c][4 * i + 2] + kv[i].z * v;
+                    S[c][4 * i + 3] = av[i].w * S[c][4 * i + 3] + kv[i].w * v;
+                    acc += qv[i].x * S[c][4 * i];
+                    acc += qv[i].y * S[c][4 * i + 1];
+                    acc += qv[i].z * S[c][4 * i + 2];
+                    acc += qv[i].w * S[c][4 * i + 3];
+                }
+                acc = row16_sum(acc);
+                if (r == 0) o_s[t * slice + jl + c] = acc;
+            }
+        }
+        __syncthreads();
+        for (int idx = tid; idx < nt * slice; idx += threads)
+            if (j0 + idx % slice < Dv)
+                raw_out[((size_t)(t0 + idx / slice) * n_heads + head) * Dv + j0 + idx % slice] = o_s[idx];
+    }
+#pragma unroll
+    for (int c = 0; c < C; ++c)
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) {
+            const int d = r * ROWS + i, j = j0 + jl + c;
+            if (j < Dv && d < D) S_mem[(size_t)d * Dv + j] = S[c][i];
+        }
+}
+
+// alpha[n, c] = exp(logsigmoid(a2_bias[c] + sum_m a[n, m] * A2[c, m]) / tau) for every token n and key channel c of all
+// heads: a thread a channel, eight tokens a workgroup (their low-rank inputs staged in LDS, a channel's row of A2
+// read once for the eight).
+#define GLA_DECAY_TOKENS 8
+template <typename T>
+__global__ __launch_bounds__(256) void gla_decay_kernel(const T* __restrict__ proj, int row_stride, int a_col,
+                                                        const T* __restrict__ a2, const float* __restrict__ a2_bias,
+                                                        float* __restrict__ alpha, int n_tokens, int channels, int rank,
+                                                        float tau_inv) {
+    extern __shared__ float a_s[];   // [GLA_DECAY_TOKENS][rank]
+    const int n0 = blockIdx.x * GLA_DECAY_TOKENS, nt = min(GLA_DECAY_TOKENS, n_tokens - n0);
+    for (int idx = threadIdx.x; idx < nt * rank; idx += blockDim.x)
+        a_s[idx] = to_float(proj[(size_t)(n0 + idx / rank) * row_stride + a_col + idx % rank]);
+    __syncthreads();
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= channels) return;
+    const T* w = a2 + (size_t)c * rank;
+    float z[GLA_DECAY_TOKENS];
+    const float b = a2_bias ? a2_bias[c] : 0.f;
+#pragma unroll
+    for (int t = 0; t < GLA_DECAY_TOKENS; ++t) z[t] = b;
+    for (int m = 0; m < rank; ++m) {
+        const float wm = to_float(w[m]);
+#pragma unroll
+        for (int t = 0; t < GLA_DECAY_TOKENS; ++t) z[t] += a_s[min(t, nt - 1) * rank + m] * wm;
+    }
+#pragma unroll
+    for (int t = 0; t < GLA_DECAY_TOKENS; ++t)
+        if (t < nt) alpha[(size_t)(n0 + t) * channels + c] = expf(log_sigmoid(z[t]) * tau_inv);
+}
+
+// y = o * rsqrt(mean(o^2) + eps) * w * silu(g) for outputs left in a float workspace: a wave a (token, head).
+template <typename T>
+__global__ __launch_bounds__(SIA_WAVE) void gla_finish_kernel(const float* __restrict__ raw, const T* __restrict__ proj,
+                                                              int row_stride, int g_col,
+                                                              const float* __restrict__ norm_w, T* __restrict__ out,
+                                                              int n_heads, int Dv, float eps) {
+    const int n = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+    const float* o = raw + ((size_t)n * n_heads + head) * Dv;
+    float ss = 0.f;
+    for (int c = lane; c < Dv; c += SIA_WAVE) ss += o[c] * o[c];
+    const float inv = rsqrtf(wave_sum(ss) / (float)Dv + eps);
+    const T* g_row = proj + (size_t)n * row_stride + g_col + head * Dv;
+    T* dst = out + ((size_t)n * n_heads + head) * Dv;
+    for (int c = lane; c < Dv; c += SIA_WAVE) {
+        const float g = to_float(g_row[c]);
+        dst[c] = from_float<T>(o[c] * inv * norm_w[c] * (g / (1.f + expf(-g))));
+    }
+}
+
 SIA_EXPORT int sia_gla_max_dims() { return 512; }
+
+// Whether a step shares a head's columns out between workgroups (and needs the outputs' part of the workspace).
+static bool gla_slices(int n_seqs, int max_q_len, int n_heads) {
+    (void)n_seqs; (void)n_heads;
+    return max_q_len > 1;
+}
+
+// Floats of workspace a step of n_tokens needs: the decays [tokens, heads, D], and the raw outputs
+// [tokens, heads, Dv] of a step whose heads' columns are shared out.
+SIA_EXPORT long long sia_gla_workspace(int n_tokens, int n_seqs, int max_q_len, int n_heads, int D, int Dv) {
+    return (long long)n_tokens * n_heads * D + (gla_slices(n_seqs, max_q_len, n_heads) ? (long long)n_tokens * n_heads * Dv : 0);
+}
 
 SIA_EXPORT int sia_gla_recurrent(const void* proj, int row_stride, int q_col, int k_col, int v_col, int g_col, int a_col,
                                  const void* a2, const float* a2_bias, const float* norm_w, float* state,
                                  const int* cu_q, const int* slots, void* out, int n_seqs, int max_q_len, int n_heads,
                                  int D, int Dv, int rank, float tau, float q_scale, float eps, int dtype,
-                                 hipStream_t stream) {
+                                 float* workspace, int n_tokens, hipStream_t stream) {
     if (n_seqs <= 0) return 0;
     if (D <= 0 || Dv <= 0 || D > 512 || Dv > 512 || rank <= 0 || rank > 1024 || n_heads <= 0 || n_heads > 65535 ||
-        !(tau > 0.f) || !state || !norm_w)
+        !(tau > 0.f) || !state || !norm_w || !workspace || n_tokens <= 0)
         return SIA_BAD_ARGUMENT;
+    float* alpha = workspace;
+    float* raw_space = workspace + (size_t)n_tokens * n_heads * D;
+    {
+        const int channels = n_heads * D;
+        dim3 dgrid((n_tokens + GLA_DECAY_TOKENS - 1) / GLA_DECAY_TOKENS, (channels + 255) / 256), dblock(256);
+        const size_t lds = (size_t)GLA_DECAY_TOKENS * rank * sizeof(float);
+        if (dtype == SIA_F32)
+            hipLaunchKernelGGL(gla_decay_kernel<float>, dgrid, dblock, lds, stream, (const float*)proj, row_stride, a_col,
+                               (const float*)a2, a2_bias, alpha, n_tokens, channels, rank, 1.f / tau);
+        else if (dtype == SIA_BF16)
+            hipLaunchKernelGGL(gla_decay_kernel<bf16_t>, dgrid, dblock, lds, stream, (const bf16_t*)proj, row_stride,
+                               a_col, (const bf16_t*)a2, a2_bias, alpha, n_tokens, channels, rank, 1.f / tau);
+        else
+            return SIA_BAD_ARGUMENT;
+    }
+    // columns a workgroup: all of a head's, or with a workspace a slice of them, as narrow as it takes to fill the chip
+    int slice = Dv;
+    const bool prompt = gla_slices(n_seqs, max_q_len, n_heads);
+    if (prompt)
+        while (slice > 8 && (long long)n_seqs * n_heads * ((Dv + slice - 1) / slice) < 256) slice = (slice + 1) / 2;
+    const bool sliced = slice < Dv;
     // lanes a column: the largest power of two that keeps the workgroup within 512 threads and a wave's columns whole
     int R = 1;
-    while (R * 2 <= SIA_WAVE && Dv * R * 2 <= 512 && R * 2 <= D) R *= 2;
+    while (R * 2 <= SIA_WAVE && slice * R * 2 <= 512 && R * 2 <= D) R *= 2;
     const int rows = (D + R - 1) / R;
     if (rows > 128) return SIA_BAD_ARGUMENT;
-    const int threads = ((Dv * R + SIA_WAVE - 1) / SIA_WAVE) * SIA_WAVE;
+    const int threads = ((slice * R + SIA_WAVE - 1) / SIA_WAVE) * SIA_WAVE;
     int TB = max_q_len >= 16 ? 16 : (max_q_len >= 4 ? 4 : 1);
-    auto bytes = [&](int tb) { return (size_t)tb * (3 * D + 3 * Dv + rank) * sizeof(float); };
+    auto bytes = [&](int tb) { return (size_t)tb * (3 * D + 3 * Dv) * sizeof(float); };
     while (TB > 1 && bytes(TB) > 60 * 1024) TB /= 2;
     if (bytes(TB) > 60 * 1024) return SIA_BAD_ARGUMENT;
-    dim3 grid(n_seqs, n_heads), block(threads);
+    dim3 grid(n_seqs, n_heads, (Dv + slice - 1) / slice), block(threads);
+    // the walk with requests a block ahead, where its pieces are aligned and fit its registers.  (Its workgroups take
+    // as many columns as their threads hold whatever the step: the waves of a workgroup share the staged tokens, and
+    // what bounds the walk is a wave's own chain of tokens, not the number of workgroups.)
+    const int w_cols = 2;
+    const int w_slice = GLA_WALK_THREADS / 16 * w_cols;
+    const int w_rows = (D + 15) / 16;
+    const int w_rows_t = w_rows <= 4 ? 4 : w_rows <= 8 ? 8 : w_rows <= 16 ? 16 : 32;
+    const size_t w_lds = (size_t)GLA_WALK_TOKENS * (3 * 16 * w_rows_t + 2 * w_slice) * sizeof(float);
+    const bool ahead = prompt && dtype == SIA_BF16 && D % 8 == 0 && row_stride % 8 == 0 && q_col % 8 == 0 &&
+                       k_col % 8 == 0 && ((uintptr_t)proj % 16) == 0 &&
+                       GLA_WALK_TOKENS * (D / 8) <= 4 * GLA_WALK_THREADS && w_lds <= 60 * 1024 && w_rows_t <= 16;
+    float* raw = (sliced || ahead) ? raw_space : nullptr;
+    if (ahead) {
+        dim3 wgrid(n_seqs, n_heads, (Dv + w_slice - 1) / w_slice), wblock(GLA_WALK_THREADS);
+#define WALK(ROWS, COLS)                                                                                             \
+    hipLaunchKernelGGL((gla_walk_kernel<ROWS, COLS>), wgrid, wblock, w_lds, stream, (const bf16_t*)proj, row_stride, \
+                       q_col, k_col, v_col, alpha, state, cu_q, slots, n_heads, D, Dv, q_scale, raw)
+        if (w_cols == 2) {
+            if (w_rows_t == 4) WALK(4, 2);
+            else if (w_rows_t == 8) WALK(8, 2);
+            else WALK(16, 2);
+        } else {
+            if (w_rows_t == 4) WALK(4, 4);
+            else if (w_rows_t == 8) WALK(8, 4);
+            else WALK(16, 4);
+        }
+#undef WALK
+    } else {
 #define LAUNCH(T, ROWS)                                                                                              \
     hipLaunchKernelGGL((gla_recurrent_kernel<T, ROWS>), grid, block, bytes(TB), stream, (const T*)proj, row_stride,  \
-                       q_col, k_col, v_col, g_col, a_col, (const T*)a2, a2_bias, norm_w, state, cu_q, slots, (T*)out, \
-                       n_heads, D, Dv, rank, R, TB, 1.f / tau, q_scale, eps)
+                       q_col, k_col, v_col, g_col, alpha, norm_w, state, cu_q, slots, (T*)out, n_heads, D, Dv, R, TB,   \
+                       q_scale, eps, slice, raw)
 #define PICK(T)                                                                                                      \
     do {                                                                                                             \
         if (rows <= 4) LAUNCH(T, 4);                                                                                 \
@@ -149,5 +439,15 @@ SIA_EXPORT int sia_gla_recurrent(const void* proj, int row_stride, int q_col, in
     else return SIA_BAD_ARGUMENT;
 #undef PICK
 #undef LAUNCH
+    }
+    if (raw) {
+        dim3 fgrid(n_tokens, n_heads), fblock(SIA_WAVE);
+        if (dtype == SIA_F32)
+            hipLaunchKernelGGL(gla_finish_kernel<float>, fgrid, fblock, 0, stream, raw, (const float*)proj, row_stride,
+                               g_col, norm_w, (float*)out, n_heads, Dv, eps);
+        else
+            hipLaunchKernelGGL(gla_finish_kernel<bf16_t>, fgrid, fblock, 0, stream, raw, (const bf16_t*)proj, row_stride,
+                               g_col, norm_w, (bf16_t*)out, n_heads, Dv, eps);
+    }
     return SIA_LAUNCH_CHECK();
 }

@@ -43,9 +43,13 @@ _SIGNATURES = {
     "sia_gla_max_dims": [],
     "sia_gla_recurrent": [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
                           _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float,
-                          _c_int, _c_ptr],
+                          _c_int, _c_ptr, _c_int, _c_ptr],
+    "sia_gla_workspace": [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int],
     "sia_moe_route": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_moe_gate_up": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "sia_moe_tiled_workspace": [_c_int, _c_int, _c_int, _c_int, _c_int],
+    "sia_moe_tiled": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
     "sia_moe_down": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int,
                      _c_int, _c_ptr],
     "sia_gemm_skinny_act": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr],
@@ -179,6 +183,9 @@ class HipKernels:
         self.core = build.load_library("core")
         _bind(self.core, _SIGNATURES)
         self.core.sia_sample_workspace_bytes.restype = ctypes.c_longlong
+        self.core.sia_gla_workspace.restype = ctypes.c_longlong
+        self.core.sia_moe_tiled_workspace.restype = ctypes.c_longlong
+        self.tiled_experts = True        # many slots in bfloat16: experts' products on the matrix cores, slots sorted by expert
         self._attn_libs = {}
         # the short way to the current stream's handle, where this torch has it (a few microseconds less a launch)
         self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -464,10 +471,20 @@ class HipKernels:
         if not (0 < key_dim <= limit and 0 < value_dim <= limit):
             raise KernelError(f"head sizes {key_dim} x {value_dim} are outside what the kernel takes (up to {limit})")
         out = torch.empty((n, n_heads * value_dim), dtype=proj.dtype, device=proj.device)
+        # float scratch for the decays and, where a prompt's step shares a head's columns out between workgroups, for
+        # their raw outputs (kept with the step: its layers run in turn)
+        floats = self.core.sia_gla_workspace(n, ctx.n_seqs, ctx.max_q_len, n_heads, key_dim, value_dim)
+        workspace = getattr(ctx, "recurrent_workspace", None)
+        if workspace is None or workspace.numel() < floats:
+            workspace = torch.empty((floats,), dtype=torch.float32, device=proj.device)
+            try:
+                ctx.recurrent_workspace = workspace
+            except AttributeError:
+                pass
         self._check(self.core.sia_gla_recurrent(
             _ptr(proj), width, q, k, v, g, a, _ptr(a2), _ptr(a2_bias), _ptr(norm_weight), _ptr(state), _ptr(ctx.cu_q),
             _ptr(ctx.state_slots), _ptr(out), ctx.n_seqs, ctx.max_q_len, n_heads, key_dim, value_dim, rank, float(tau),
-            float(q_scale), float(eps), _DT[proj.dtype], self._stream()), "gla_recurrent")
+            float(q_scale), float(eps), _DT[proj.dtype], _ptr(workspace), n, self._stream()), "gla_recurrent")
         return out
 
     def check_recurrent_geometry(self, key_dim: int, value_dim: int) -> None:
@@ -514,6 +531,16 @@ class HipKernels:
             raise KernelError("a shared expert's gate comes with its output")
         act = torch.empty((n * top, ff), dtype=h.dtype, device=h.device)
         out = torch.empty((n, width), dtype=h.dtype, device=h.device)
+        ints = self.core.sia_moe_tiled_workspace(n, top, experts, width, ff) if (
+            self.tiled_experts and h.dtype == torch.bfloat16) else 0
+        if ints:
+            workspace = torch.empty((ints,), dtype=torch.int32, device=h.device)
+            y = torch.empty((n * top, width), dtype=h.dtype, device=h.device)
+            self._check(self.core.sia_moe_tiled(
+                _ptr(h), _ptr(w_gate_up), _ptr(w_down), _ptr(ids), _ptr(weights), _ptr(shared), _ptr(shared_gate),
+                gate_stride, _ptr(act), _ptr(y), _ptr(out), _ptr(workspace), n, width, ff, top, experts,
+                self._stream()), "moe_tiled")
+            return out
         self._check(self.core.sia_moe_gate_up(_ptr(h), _ptr(w_gate_up), _ptr(ids), _ptr(act), n, width, ff, top,
                                               _DT[h.dtype], self._stream()), "moe_gate_up")
         self._check(self.core.sia_moe_down(_ptr(act), _ptr(w_down), _ptr(ids), _ptr(weights), _ptr(shared),

@@ -69,9 +69,15 @@ CONFIGS = {
           "loop": {"start": 0, "stop": 2, "times": 1},
           "layers": [_layer(_att(2, 2, 24, 24, 0.25, (1.0, 3)), None),
                      _layer(_gla(2, 16, 24, 2.0, 4), _moe(3, 2, 16, 8))]},
+    # sizes that are multiples of nothing the kernels like: every vector path has to step aside
+    "e": {"architecture": "Mogisun", "vocab": 131, "width": 100, "norm": {"eps": 2e-6}, "logit_scale": 1.3,
+          "logit_softcap": 9.0, "loop": {"start": 1, "stop": 2, "times": 2},
+          "layers": [_layer(_att(5, 5, 20, 12, 0.4, (0.2, 5)), _moe(7, 2, 36, 20)),
+                     _layer(_gla(3, 12, 20, 3.0, 7), _dense(52)),
+                     _layer(_att(3, 1, 12, 28, 0.3), _moe(2, 1, 10))]},
 }
 
-PAGE_SIZE = {"a": 8, "b": 16, "c": 16, "d": 4}
+PAGE_SIZE = {"a": 8, "b": 16, "c": 16, "d": 4, "e": 16}
 
 
 def all_experts(cfg):

@@ -178,7 +178,7 @@ def test_the_residual_after_every_run_of_a_layer_is_the_plain_one(folders):
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "d", "e"])
 def test_whole_prompt_then_token_by_token(folders, backend, name):
     folder = folder_for(folders, name, backend)
     runner, cache = M.make_runner(folder, backend, M.PAGE_SIZE[name], 40)
@@ -195,7 +195,7 @@ def test_whole_prompt_then_token_by_token(folders, backend, name):
 
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("name,sizes", [("a", [2, 5, 23, 1, 24, 3]), ("b", [19, 2, 2, 40, 1, 7]), ("c", [50, 17, 2, 33, 64]),
-                                        ("d", [3, 2, 2, 31])])
+                                        ("d", [3, 2, 2, 31]), ("e", [7, 2, 45, 1, 16])])
 def test_portions_cut_anywhere_down_to_two_tokens(folders, backend, name, sizes):
     folder = folder_for(folders, name, backend)
     runner, cache = M.make_runner(folder, backend, M.PAGE_SIZE[name], 40)

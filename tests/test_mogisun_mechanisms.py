@@ -234,16 +234,20 @@ def test_the_router_picks_the_largest_logits_and_weighs_them_among_themselves(ba
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("experts,top,width,ff,shared", [(5, 1, 96, 40, False), (8, 3, 128, 24, True), (4, 2, 50, 17, True),
-                                                         (6, 6, 64, 128, False)])
-def test_experts_weighted_and_summed_with_a_shared_one(backend, experts, top, width, ff, shared):
+@pytest.mark.parametrize("experts,top,width,ff,shared,n", [
+    (5, 1, 96, 40, False, 11), (8, 3, 128, 24, True, 11), (4, 2, 50, 17, True, 11), (6, 6, 64, 128, False, 11),
+    # steps of many slots, which the GPU sorts by expert and multiplies in tiles: tiles that are not full, experts
+    # nobody chose, columns that do not fill a workgroup's share
+    (8, 2, 160, 96, True, 203), (16, 1, 64, 32, False, 70), (3, 3, 128, 288, True, 64)])
+def test_experts_weighted_and_summed_with_a_shared_one(backend, experts, top, width, ff, shared, n):
     k, dev, dtype, tol = setup(backend)
     g = torch.Generator().manual_seed(ff)
-    n = 11
     h, h64 = lowered(rnd(g, n, width), dtype, dev)
     w1, w1_64 = lowered(rnd(g, experts, 2 * ff, width, std=0.1), dtype, dev)
     w2, w2_64 = lowered(rnd(g, experts, width, ff, std=0.1), dtype, dev)
     ids = torch.stack([torch.randperm(experts, generator=g)[:top] for _ in range(n)]).to(torch.int32)
+    if experts == 16:
+        ids = ids % 5          # most experts are chosen by nobody
     weights = torch.softmax(rnd(g, n, top), -1).float()
     sh = sg = sh64 = sg64 = None
     if shared:
