@@ -21,12 +21,18 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
     __shared__ float logit_s[MOE_MAX_EXPERTS];
     const int n = blockIdx.x, wave = threadIdx.x / SIA_WAVE, lane = threadIdx.x % SIA_WAVE;
     const T* x = h + (size_t)n * width;
+    // a wave an expert at a time; four independent runs of loads a lane, so that a row's latency is paid once
     for (int e = wave; e < n_experts; e += blockDim.x / SIA_WAVE) {
         const float* w = router + (size_t)e * width;
-        float acc = 0.f;
-        for (int i = lane; i < width; i += SIA_WAVE) acc += to_float(x[i]) * w[i];
-        acc = wave_sum(acc);
-        if (lane == 0) logit_s[e] = acc;
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        int i = lane;
+        for (; i + 3 * SIA_WAVE < width; i += 4 * SIA_WAVE) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc[u] += to_float(x[i + u * SIA_WAVE]) * w[i + u * SIA_WAVE];
+        }
+        for (; i < width; i += SIA_WAVE) acc[0] += to_float(x[i]) * w[i];
+        const float total = wave_sum((acc[0] + acc[1]) + (acc[2] + acc[3]));
+        if (lane == 0) logit_s[e] = total;
     }
     __syncthreads();
     if (wave != 0) return;

@@ -54,7 +54,7 @@ def context(device, q_lens, slots):
 
 # ---------------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("hidden,extra", [(96, 0), (192, 24), (50, 3), (1024, 8)])
+@pytest.mark.parametrize("hidden,extra", [(96, 0), (176, 24), (50, 3), (1024, 8)])
 def test_gated_sum_into_the_residual_and_the_norm_after_it(backend, hidden, extra):
     k, dev, dtype, tol = setup(backend)
     g = torch.Generator().manual_seed(hidden)
@@ -119,7 +119,7 @@ def test_the_query_temperature_steps_where_the_formula_says():
 
 # ---------------------------------------------------------------------------------------------------------------
 GLA_SHAPES = [(3, 24, 40, 5, 4.0), (1, 8, 8, 3, 1.0), (2, 64, 64, 8, 16.0), (2, 128, 128, 16, 8.0), (2, 256, 48, 33, 2.0),
-              (5, 48, 32, 16, 16.0), (1, 40, 200, 2, 0.5)]
+              (5, 56, 24, 12, 6.0), (1, 40, 200, 2, 0.5)]
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
@@ -210,7 +210,7 @@ def test_linear_attention_remembers_one_token_over_a_long_decode(backend):
 
 # ---------------------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("backend", BACKENDS)
-@pytest.mark.parametrize("experts,top,width", [(5, 1, 96), (8, 3, 128), (12, 2, 50), (7, 7, 64), (70, 6, 128)])
+@pytest.mark.parametrize("experts,top,width", [(5, 1, 96), (8, 3, 128), (11, 2, 50), (7, 7, 64), (70, 6, 128)])
 def test_the_router_picks_the_largest_logits_and_weighs_them_among_themselves(backend, experts, top, width):
     k, dev, dtype, tol = setup(backend)
     g = torch.Generator().manual_seed(experts)
