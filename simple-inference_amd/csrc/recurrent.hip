@@ -163,77 +163,84 @@ __global__ __launch_bounds__(GLA_WALK_THREADS) void gla_walk_kernel(
             S[c][i] = (j < Dv && d < D) ? S_mem[(size_t)d * Dv + j] : 0.f;
         }
     const int d8 = D / 8, d4 = D / 4;
-    uint4 rq[4], rk[4];
-    float4 ra[8];
-    float rv[TB * slice / threads];     // a block's values: 32 tokens x 16 C columns over 256 threads
-    auto request = [&](int t0) {   // the block's pieces into registers; pieces beyond the sequence's end are not read
-        const int nt = min(TB, last - t0);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int idx = tid + i * threads;
-            if (idx < nt * d8) {
-                const bf16_t* row = proj + (size_t)(t0 + idx / d8) * row_stride + head * D + (idx % d8) * 8;
-                rq[i] = *reinterpret_cast<const uint4*>(row + q_col);
-                rk[i] = *reinterpret_cast<const uint4*>(row + k_col);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int idx = tid + i * threads;
-            if (idx < nt * d4)
-                ra[i] = *reinterpret_cast<const float4*>(alpha + ((size_t)(t0 + idx / d4) * n_heads + head) * D + (idx % d4) * 4);
-        }
-#pragma unroll
-        for (int i = 0; i < TB * slice / threads; ++i) {
-            const int idx = tid + i * threads;
-            if (idx < nt * slice && j0 + idx % slice < Dv)
-                rv[i] = bf16_to_float(proj[(size_t)(t0 + idx / slice) * row_stride + v_col + head * Dv + j0 + idx % slice]);
-        }
-    };
-    auto deposit = [&](int t0) {
-        const int nt = min(TB, last - t0);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int idx = tid + i * threads;
-            if (idx < nt * d8) {
-                const int base = (idx / d8) * Dp, d0 = (idx % d8) * 8;
-                // two 16-bit halves of a word are rows d and d + 1; no arrays, so that all of it stays in registers
-#define GLA_PUT(word_q, word_k, d)                                                                \
-    do {                                                                                          \
-        const int p0 = base + place(d), p1 = base + place((d) + 1);                               \
-        q_s[p0] = __uint_as_float((word_q) << 16) * q_scale;                                      \
-        q_s[p1] = __uint_as_float((word_q) & 0xffff0000u) * q_scale;                              \
-        k_s[p0] = __uint_as_float((word_k) << 16);                                                \
-        k_s[p1] = __uint_as_float((word_k) & 0xffff0000u);                                        \
+    // What is on its way from memory is held in named registers, and the two steps below are written out piece by
+    // piece: arrays indexed in loops ended up in scratch memory here, and a wave then waited for every piece twice.
+    static_assert(TB * slice / threads == 4, "four values a thread and block");
+    uint4 rq0, rq1, rq2, rq3, rk0, rk1, rk2, rk3;
+    float4 ra0, ra1, ra2, ra3, ra4, ra5, ra6, ra7;
+    float rv0, rv1, rv2, rv3;
+    // pieces beyond the block's end repeat its last piece (every load is issued, none is conditional)
+#define GLA_REQ_QK(i, Q, K)                                                                          \
+    do {                                                                                             \
+        const int idx = min(tid + (i) * threads, rnt * d8 - 1);                                       \
+        const bf16_t* row = proj + (size_t)(rt0 + idx / d8) * row_stride + head * D + (idx % d8) * 8; \
+        Q = *reinterpret_cast<const uint4*>(row + q_col);                                            \
+        K = *reinterpret_cast<const uint4*>(row + k_col);                                            \
     } while (0)
-                GLA_PUT(rq[i].x, rk[i].x, d0);
-                GLA_PUT(rq[i].y, rk[i].y, d0 + 2);
-                GLA_PUT(rq[i].z, rk[i].z, d0 + 4);
-                GLA_PUT(rq[i].w, rk[i].w, d0 + 6);
-#undef GLA_PUT
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int idx = tid + i * threads;
-            if (idx < nt * d4) {
-                const int base = (idx / d4) * Dp, d0 = (idx % d4) * 4;   // four rows of one lane (ROWS is a multiple of 4)
-                *reinterpret_cast<float4*>(al_s + base + place(d0)) = ra[i];
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < TB * slice / threads; ++i) {
-            const int idx = tid + i * threads;
-            if (idx < nt * slice) v_s[idx] = (j0 + idx % slice < Dv) ? rv[i] : 0.f;
-        }
-    };
+#define GLA_REQ_A(i, A)                                                                              \
+    do {                                                                                             \
+        const int idx = min(tid + (i) * threads, rnt * d4 - 1);                                       \
+        A = *reinterpret_cast<const float4*>(alpha + ((size_t)(rt0 + idx / d4) * n_heads + head) * D + (idx % d4) * 4); \
+    } while (0)
+#define GLA_REQ_V(i, V)                                                                              \
+    do {                                                                                             \
+        const int idx = min(tid + (i) * threads, rnt * slice - 1);                                    \
+        V = bf16_to_float(proj[(size_t)(rt0 + idx / slice) * row_stride + v_col + head * Dv +         \
+                               min(j0 + idx % slice, Dv - 1)]);                                      \
+    } while (0)
+#define GLA_REQUEST(T0)                                                                              \
+    do {                                                                                             \
+        const int rt0 = (T0), rnt = min(TB, last - rt0);                                                \
+        GLA_REQ_QK(0, rq0, rk0); GLA_REQ_QK(1, rq1, rk1); GLA_REQ_QK(2, rq2, rk2); GLA_REQ_QK(3, rq3, rk3); \
+        GLA_REQ_A(0, ra0); GLA_REQ_A(1, ra1); GLA_REQ_A(2, ra2); GLA_REQ_A(3, ra3);                  \
+        GLA_REQ_A(4, ra4); GLA_REQ_A(5, ra5); GLA_REQ_A(6, ra6); GLA_REQ_A(7, ra7);                  \
+        GLA_REQ_V(0, rv0); GLA_REQ_V(1, rv1); GLA_REQ_V(2, rv2); GLA_REQ_V(3, rv3);                  \
+    } while (0)
+    // two 16-bit halves of a word are rows d and d + 1
+#define GLA_PUT(word_q, word_k, d)                                                                   \
+    do {                                                                                             \
+        const int p0 = base + place(d), p1 = base + place((d) + 1);                                  \
+        q_s[p0] = __uint_as_float((word_q) << 16) * q_scale;                                         \
+        q_s[p1] = __uint_as_float((word_q) & 0xffff0000u) * q_scale;                                 \
+        k_s[p0] = __uint_as_float((word_k) << 16);                                                   \
+        k_s[p1] = __uint_as_float((word_k) & 0xffff0000u);                                           \
+    } while (0)
+#define GLA_DEP_QK(i, Q, K)                                                                          \
+    do {                                                                                             \
+        const int idx = tid + (i) * threads;                                                         \
+        if (idx < dnt * d8) {                                                                         \
+            const int base = (idx / d8) * Dp, d0 = (idx % d8) * 8;                                   \
+            GLA_PUT(Q.x, K.x, d0);                                                                   \
+            GLA_PUT(Q.y, K.y, d0 + 2);                                                               \
+            GLA_PUT(Q.z, K.z, d0 + 4);                                                               \
+            GLA_PUT(Q.w, K.w, d0 + 6);                                                               \
+        }                                                                                            \
+    } while (0)
+#define GLA_DEP_A(i, A)                                                                              \
+    do {   /* four rows of one lane (ROWS is a multiple of 4) */                                     \
+        const int idx = tid + (i) * threads;                                                         \
+        if (idx < dnt * d4) *reinterpret_cast<float4*>(al_s + (idx / d4) * Dp + place((idx % d4) * 4)) = A; \
+    } while (0)
+#define GLA_DEP_V(i, V)                                                                              \
+    do {                                                                                             \
+        const int idx = tid + (i) * threads;                                                         \
+        if (idx < dnt * slice) v_s[idx] = (j0 + idx % slice < Dv) ? V : 0.f;                          \
+    } while (0)
+#define GLA_DEPOSIT(T0)                                                                              \
+    do {                                                                                             \
+        const int dnt = min(TB, last - (T0));                                                         \
+        GLA_DEP_QK(0, rq0, rk0); GLA_DEP_QK(1, rq1, rk1); GLA_DEP_QK(2, rq2, rk2); GLA_DEP_QK(3, rq3, rk3); \
+        GLA_DEP_A(0, ra0); GLA_DEP_A(1, ra1); GLA_DEP_A(2, ra2); GLA_DEP_A(3, ra3);                  \
+        GLA_DEP_A(4, ra4); GLA_DEP_A(5, ra5); GLA_DEP_A(6, ra6); GLA_DEP_A(7, ra7);                  \
+        GLA_DEP_V(0, rv0); GLA_DEP_V(1, rv1); GLA_DEP_V(2, rv2); GLA_DEP_V(3, rv3);                  \
+    } while (0)
     // One round before the first block only requests it (each of the two steps is written once, so that the pieces
     // on their way stay in registers).
     for (int t0 = first - TB; t0 < last; t0 += TB) {
         const int nt = min(TB, last - t0);
-        if (t0 >= first) deposit(t0);
+        if (t0 >= first) GLA_DEPOSIT(t0);
         __syncthreads();   // in the first round: the zeros are in place before the first pieces land on them
-        if (t0 + TB < last) request(t0 + TB);
+        if (t0 + TB < last) GLA_REQUEST(t0 + TB);
         if (t0 < first) continue;   // uniform
         // a token's q, k and decays are read from LDS while the token before is worked on
         float4 qn[ROWS / 4], kn[ROWS / 4], an[ROWS / 4];
@@ -287,6 +294,16 @@ __global__ __launch_bounds__(GLA_WALK_THREADS) void gla_walk_kernel(
             if (j < Dv && d < D) S_mem[(size_t)d * Dv + j] = S[c][i];
         }
 }
+
+#undef GLA_REQ_QK
+#undef GLA_REQ_A
+#undef GLA_REQ_V
+#undef GLA_REQUEST
+#undef GLA_PUT
+#undef GLA_DEP_QK
+#undef GLA_DEP_A
+#undef GLA_DEP_V
+#undef GLA_DEPOSIT
 
 // alpha[n, c] = exp(logsigmoid(a2_bias[c] + sum_m a[n, m] * A2[c, m]) / tau) for every token n and key channel c of all
 // heads: a thread a channel, eight tokens a workgroup (their low-rank inputs staged in LDS, a channel's row of A2
@@ -410,15 +427,9 @@ SIA_EXPORT int sia_gla_recurrent(const void* proj, int row_stride, int q_col, in
 #define WALK(ROWS, COLS)                                                                                             \
     hipLaunchKernelGGL((gla_walk_kernel<ROWS, COLS>), wgrid, wblock, w_lds, stream, (const bf16_t*)proj, row_stride, \
                        q_col, k_col, v_col, alpha, state, cu_q, slots, n_heads, D, Dv, q_scale, raw)
-        if (w_cols == 2) {
-            if (w_rows_t == 4) WALK(4, 2);
-            else if (w_rows_t == 8) WALK(8, 2);
-            else WALK(16, 2);
-        } else {
-            if (w_rows_t == 4) WALK(4, 4);
-            else if (w_rows_t == 8) WALK(8, 4);
-            else WALK(16, 4);
-        }
+        if (w_rows_t == 4) WALK(4, 2);
+        else if (w_rows_t == 8) WALK(8, 2);
+        else WALK(16, 2);
 #undef WALK
     } else {
 #define LAUNCH(T, ROWS)                                                                                              \
