@@ -9,7 +9,7 @@
 //     normed and only the residual is updated (the sum is wanted by itself: where a stream is re-mixed).  With
 //     ``rows`` only those rows are normed and the residual is left as it was.
 //   bias:                   y[n, :] += b                                in place
-//   head gate:              out[n, h, :] *= sigmoid(logit[n, h])        one number per token and head
+//   head gate:              out[n, h, :] *= sigmoid(logit[n, h])        a scalar for every token and head
 //   side by side:           out[n, :] = [T(a[n, :]), T(b[n, :])]        two float streams lowered into one row
 //   scale + soft cap:       z <- cap * tanh(z * scale / cap)            (cap <= 0: z <- z * scale), in place, float
 #include "common.h"

@@ -30,7 +30,7 @@ Further forms, each switched on by a parameter of its own and free to combine:
 * ``qk_norm`` with ``"gain": False``: the same division by the root mean square without learned gains.
 * ``q_temp`` (``{"coef": c, "every": n}``): a query at position ``p`` is multiplied by
   ``1 + c * ln(floor((p + 1) / n) + 1)`` after its norm, so late queries score more sharply.
-* ``out_gate``: head ``h``'s output is multiplied by ``sigmoid((G x)_h)``, one number per token and head, ``G
+* ``out_gate``: head ``h``'s output is multiplied by ``sigmoid((G x)_h)``, a scalar for every token and head, ``G
   [Hq, H]`` reading the mixer's own input; its rows ride at the end of the stacked projection.
 * ``o_bias``: the output projection has a bias; it is handed on with the result (``BiasedDelta``) so that the sum
   into the residual can take it in passing.

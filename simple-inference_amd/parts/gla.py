@@ -9,10 +9,10 @@ For a token with input ``h`` (``H`` heads, key width ``D``, value width ``Dv``):
     o = S^T q                                 the state already holds this token
     y = Wo (concat_h(o_h / rms(o_h) * w) * silu(Wg h))
 
-The state starts at zero, is float32 in both modes and lives in the request's state slot (one per run of the
-layer); the cache manager hands it in as ``cache.state``.  A sequence's tokens must arrive in order, which the step
-function guarantees.  All input projections (q, k, v, g and the low-rank ``A1``) are one stacked matrix; the decays
-(``A2``, bias, log-sigmoid, the power) are computed inside the recurrence's kernel, in float.
+A request's state is all zeros before its first token, float32 in both modes, and kept in the request's state slot
+(one per run of the layer); the cache manager hands it in as ``cache.state``.  A sequence's tokens must arrive in
+order, which the step function guarantees.  All input projections (q, k, v, g and the low-rank ``A1``) are one
+stacked matrix; the decays (``A2``, bias, log-sigmoid, the power) are the kernels' business, in float.
 
 The rank of the low-rank pair is whatever the checkpoint's tensors have, unless ``decay_rank`` names it.
 """

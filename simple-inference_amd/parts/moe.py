@@ -4,7 +4,7 @@
     chosen: the ``top`` largest logits (ties: the lower index); weights: softmax over the chosen logits alone
     y = sum_k weight_k * W2_e (silu(Wg_e h) * (Wu_e h))        e = the k-th chosen expert; experts have no biases
     y += sigmoid(s . h) * Ws2 (silu(Wsg h) * (Wsu h))          a shared expert every token runs, if the layer has one,
-                                                              scaled by one number per token
+                                                              scaled by a scalar of the token's own
 
 The experts' matrices are stacked at load (``[E, 2 ff, hidden]`` with the gate rows first, ``[E, hidden, ff]``); the
 shared expert's gate and up rows and its scalar gate are one stacked matrix.  Routing happens on the device: no
