@@ -363,10 +363,11 @@ static bool gla_slices(int n_seqs, int max_q_len, int n_heads) {
     return max_q_len > 1;
 }
 
-// Floats of workspace a step of n_tokens needs: the decays [tokens, heads, D], and the raw outputs
+// Floats of workspace a step of n_tokens needs: the decays [tokens, heads, D], and room for the raw outputs
 // [tokens, heads, Dv] of a step whose heads' columns are shared out.
 SIA_EXPORT long long sia_gla_workspace(int n_tokens, int n_seqs, int max_q_len, int n_heads, int D, int Dv) {
-    return (long long)n_tokens * n_heads * D + (gla_slices(n_seqs, max_q_len, n_heads) ? (long long)n_tokens * n_heads * Dv : 0);
+    (void)n_seqs; (void)max_q_len;
+    return (long long)n_tokens * n_heads * D + (long long)n_tokens * n_heads * Dv;
 }
 
 SIA_EXPORT int sia_gla_recurrent(const void* proj, int row_stride, int q_col, int k_col, int v_col, int g_col, int a_col,
@@ -398,12 +399,18 @@ SIA_EXPORT int sia_gla_recurrent(const void* proj, int row_stride, int q_col, in
     const bool prompt = gla_slices(n_seqs, max_q_len, n_heads);
     if (prompt)
         while (slice > 8 && (long long)n_seqs * n_heads * ((Dv + slice - 1) / slice) < 256) slice = (slice + 1) / 2;
-    const bool sliced = slice < Dv;
-    // lanes a column: the largest power of two that keeps the workgroup within 512 threads and a wave's columns whole
-    int R = 1;
-    while (R * 2 <= SIA_WAVE && slice * R * 2 <= 512 && R * 2 <= D) R *= 2;
-    const int rows = (D + R - 1) / R;
+    // lanes a column: the largest power of two that keeps the workgroup within 512 threads and a wave's columns whole;
+    // a state too tall for the rows a lane can keep is shared out over more workgroups, whatever the step
+    int R = 1, rows = D;
+    for (;;) {
+        R = 1;
+        while (R * 2 <= SIA_WAVE && slice * R * 2 <= 512 && R * 2 <= D) R *= 2;
+        rows = (D + R - 1) / R;
+        if (rows <= 128 || slice <= 1) break;
+        slice = (slice + 1) / 2;
+    }
     if (rows > 128) return SIA_BAD_ARGUMENT;
+    const bool sliced = slice < Dv;
     const int threads = ((slice * R + SIA_WAVE - 1) / SIA_WAVE) * SIA_WAVE;
     int TB = max_q_len >= 16 ? 16 : (max_q_len >= 4 ? 4 : 1);
     auto bytes = [&](int tb) { return (size_t)tb * (3 * D + 3 * Dv) * sizeof(float); };

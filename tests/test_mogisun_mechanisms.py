@@ -119,18 +119,18 @@ def test_the_query_temperature_steps_where_the_formula_says():
 
 # ---------------------------------------------------------------------------------------------------------------
 GLA_SHAPES = [(3, 24, 40, 5, 4.0), (1, 8, 8, 3, 1.0), (2, 64, 64, 8, 16.0), (2, 128, 128, 16, 8.0), (2, 256, 48, 33, 2.0),
-              (5, 56, 24, 12, 6.0), (1, 40, 200, 2, 0.5)]
+              (5, 56, 24, 12, 6.0), (1, 40, 200, 2, 0.5), (1, 264, 512, 4, 2.0)]
 
 
 @pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("H,D,Dv,rank,tau", GLA_SHAPES)
 def test_linear_attention_carries_its_state_through_any_cut(backend, H, D, Dv, rank, tau):
     """Three sequences of unequal length in scattered slots, fed in three steps of unequal portions (one of a single
-    token, one of two): every output is the plain recurrence's over the whole sequence, and the states left in the
-    slots are its last states."""
+    token, one of two) and a last step in which each brings one token (a decode step): every output is the plain
+    recurrence's over the whole sequence, and the states left in the slots are its last states."""
     k, dev, dtype, tol = setup(backend)
     g = torch.Generator().manual_seed(H * 1000 + D)
-    lengths, slots = [37, 5, 21], [4, 0, 2]
+    lengths, slots = [38, 6, 22], [4, 0, 2]
     pad = 8                          # columns in front of q that belong to somebody else
     width = pad + 2 * H * D + 2 * H * Dv + rank
     cols = (pad, pad + H * D, pad + 2 * H * D, pad + 2 * H * D + H * Dv, pad + 2 * H * D + 2 * H * Dv)
@@ -141,10 +141,10 @@ def test_linear_attention_carries_its_state_through_any_cut(backend, H, D, Dv, r
     state[4].fill_(0.0)
     cache = LayerCache(state=state)
     eps, q_scale = 1e-5, D ** -0.5
-    cuts = [[20, 1, 16], [2, 2, 1], [1, 18, 2]]
+    cuts = [[20, 1, 16, 1], [2, 2, 1, 1], [1, 18, 2, 1]]
     got = [[] for _ in lengths]
     at = [0, 0, 0]
-    for step in range(3):
+    for step in range(4):
         order = [1, 0, 2] if step == 1 else [0, 1, 2]        # the batch's order changes from step to step
         q_lens = [cuts[s][step] for s in order]
         ctx = context(dev, q_lens, [slots[s] for s in order])
